@@ -44,7 +44,161 @@ class ModelArchConfig(BaseModel):
         return self.head_dim or (self.hidden_size // self.num_heads)
 
 
-MODEL_PRESETS: dict[str, ModelArchConfig] = {
+class RotarySpec(BaseModel):
+    """Rotary position parameters of one attention mixer: the first ``dims``
+    dimensions of each head rotate as interleaved pairs (2i, 2i+1) with
+    frequency base^(-2i/dims); ``scaling`` is the banded frequency rescale
+    (factor / low / high / original context), None = plain."""
+
+    base: float = 10000.0
+    dims: int = 0
+    scaling: Optional[dict] = None
+
+
+class BlockAttnSpec(BaseModel):
+    """Softmax attention whose causal mask is cut into aligned blocks of
+    ``mask_size`` positions (0 = plain causal). ``values_from_keys``: no value
+    projection, the values are the un-rotated keys."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    mask_size: int = 0
+    rot: RotarySpec = Field(default_factory=RotarySpec)
+    values_from_keys: bool = True
+    qk_bias: bool = True
+    head_gate: bool = True
+
+
+class DecayLinearAttnSpec(BaseModel):
+    """Linear attention with one constant decay per head:
+    S <- decay_h S + k v^T, o = S^T q."""
+
+    heads: int
+    dim: int
+    vdim: int
+    decay: List[float]
+
+
+class ParallelMixerSpec(BaseModel):
+    left: BlockAttnSpec
+    right: DecayLinearAttnSpec
+
+
+class ChannelDeltaSpec(BaseModel):
+    """Gated delta rule with a decay per head and key channel, short causal
+    convolutions of ``conv`` taps on q/k/v."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    # bottleneck widths of the two low-rank projections (decay, output gate);
+    # a checkpoint fixes them by its tensor shapes
+    decay_rank: int = 16
+    gate_rank: int = 16
+
+
+class GluSpec(BaseModel):
+    """Clamped gated-linear-unit feed-forward: g = min(gate, limit),
+    u = clamp(up, +-limit), y = g * sigmoid(alpha g) * (u + 1)."""
+
+    kind: Literal["dense"] = "dense"
+    ff: int
+    limit: float
+    alpha: float = 1.702
+
+
+class HybridLayerSpec(BaseModel):
+    type: Literal["parallel", "channel_delta"]
+    parallel: Optional[ParallelMixerSpec] = None
+    channel_delta: Optional[ChannelDeltaSpec] = None
+    mlp: Optional[GluSpec] = None
+
+
+class HybridArchConfig(BaseModel):
+    """A decoder whose layers are listed one by one, each with its own
+    sequence mixer (attention and/or recurrent) and optional feed-forward —
+    the Zutalix family. Every size comes from the checkpoint's config.json."""
+
+    arch: Literal["zutalix"] = "zutalix"
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float = 1e-6
+    layers: List[HybridLayerSpec]
+    # no rotary table: angles are computed from the position in the kernel
+    max_position_embeddings: int = 1 << 24
+    tie_word_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_checkpoint_config(cls, d: dict, shapes: Optional[dict] = None) -> "HybridArchConfig":
+        """Parse the family's config.json (keys: vocab, width, norm.eps,
+        layers[].type / .mixer / .mlp). ``shapes`` (tensor name -> shape, from
+        the safetensors header) supplies the sizes config.json leaves to the
+        tensors: the low-rank bottlenecks."""
+        layers = []
+        shapes = shapes or {}
+        for li, spec in enumerate(d["layers"]):
+            m = spec["mixer"]
+            mlp = spec.get("mlp")
+            glu = GluSpec(kind=mlp.get("kind", "dense"), ff=mlp["ff"], limit=mlp["limit"]) if mlp else None
+            if spec["type"] == "parallel":
+                le, ri = m["left"], m["right"]
+                rot = le.get("rot") or {}
+                left = BlockAttnSpec(
+                    heads=le["heads"], kv_heads=le["kv_heads"], dim=le["dim"], vdim=le["vdim"],
+                    scale=le["scale"], mask_size=(le.get("mask") or {}).get("size", 0),
+                    rot=RotarySpec(base=rot.get("base", 10000.0), dims=rot.get("dims", 0),
+                                   scaling=rot.get("scaling")),
+                )
+                right = DecayLinearAttnSpec(heads=ri["heads"], dim=ri["dim"], vdim=ri["vdim"],
+                                            decay=list(ri["decay"]))
+                layers.append(HybridLayerSpec(type="parallel", mlp=glu,
+                                              parallel=ParallelMixerSpec(left=left, right=right)))
+            elif spec["type"] == "channel_delta":
+                layers.append(HybridLayerSpec(type="channel_delta", mlp=glu, channel_delta=ChannelDeltaSpec(
+                    heads=m["heads"], kv_heads=m["kv_heads"], dim=m["dim"], vdim=m["vdim"], conv=m["conv"],
+                    decay_rank=(shapes.get(f"l{li}.mix.a1") or [16])[0],
+                    gate_rank=(shapes.get(f"l{li}.mix.g1") or [16])[0])))
+            else:
+                raise ValueError(f"unknown layer type {spec['type']!r}")
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"],
+                   rms_norm_eps=d["norm"]["eps"], layers=layers)
+
+
+def _zutalix_preset(vocab, width, n_par, heads, kv_heads, dim, mask, lin_heads, lin_dim, lin_vdim,
+                    d_heads, d_kv, d_dim, d_vdim, ff, pattern="ppd", rot_dims=None, conv=4,
+                    scaling=None) -> HybridArchConfig:
+    """Random-init presets of the family: ``pattern`` repeats over the depth
+    ('p' = parallel layer with feed-forward, 'd' = delta layer without)."""
+    import math as _math
+
+    layers = []
+    for i in range(n_par):
+        if pattern[i % len(pattern)] == "p":
+            left = BlockAttnSpec(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim,
+                                 scale=1.0 / _math.sqrt(dim), mask_size=mask,
+                                 rot=RotarySpec(base=500000.0, dims=rot_dims or dim, scaling=scaling))
+            right = DecayLinearAttnSpec(
+                heads=lin_heads, dim=lin_dim, vdim=lin_vdim,
+                decay=[_math.exp(-1.0 / (2.0 ** (1 + 2 * h))) for h in range(lin_heads)])
+            layers.append(HybridLayerSpec(type="parallel", parallel=ParallelMixerSpec(left=left, right=right),
+                                          mlp=GluSpec(ff=ff, limit=7.0)))
+        else:
+            layers.append(HybridLayerSpec(type="channel_delta", channel_delta=ChannelDeltaSpec(
+                heads=d_heads, kv_heads=d_kv, dim=d_dim, vdim=d_vdim, conv=conv,
+                decay_rank=max(8, width // 32), gate_rank=max(8, width // 32))))
+    return HybridArchConfig(vocab_size=vocab, hidden_size=width, layers=layers)
+
+
+MODEL_PRESETS: dict = {
     # Llama-3-8B — the BASELINE headline config
     "llama-3-8b": ModelArchConfig(
         arch="llama", vocab_size=128256, hidden_size=4096, intermediate_size=14336,
@@ -114,6 +268,18 @@ MODEL_PRESETS: dict[str, ModelArchConfig] = {
         max_position_embeddings=512, attention_qkv_bias=True,
         tie_word_embeddings=True,
     ),
+    # Zutalix family (listed-layer hybrid: block-local softmax attention +
+    # decayed linear attention in parallel, gated-delta layers between)
+    "tiny-zutalix": _zutalix_preset(
+        vocab=512, width=64, n_par=3, heads=4, kv_heads=2, dim=16, mask=24,
+        lin_heads=2, lin_dim=8, lin_vdim=16, d_heads=2, d_kv=1, d_dim=16, d_vdim=24, ff=96),
+    "mid-zutalix": _zutalix_preset(
+        vocab=2048, width=512, n_par=3, heads=4, kv_heads=2, dim=128, mask=256,
+        lin_heads=4, lin_dim=64, lin_vdim=128, d_heads=4, d_kv=2, d_dim=64, d_vdim=128, ff=1024),
+    # layer shapes of an 8B-class model at reduced depth (bench sizes)
+    "zutalix-8b-l6": _zutalix_preset(
+        vocab=128256, width=4096, n_par=6, heads=32, kv_heads=8, dim=128, mask=2048,
+        lin_heads=32, lin_dim=128, lin_vdim=128, d_heads=32, d_kv=16, d_dim=128, d_vdim=128, ff=14336),
 }
 
 
@@ -142,6 +308,10 @@ class EngineConfig(BaseModel):
 
     max_seq_len: int = 8192
     max_batch_size: int = 256
+    # recurrent-state slots (models with linear-attention / delta-rule /
+    # convolution state keep one slot per live sequence); None = derived
+    # from max_batch_size
+    max_state_slots: Optional[int] = None
 
     # embeddings.create backend: "token_mean" mean-pools the model's token
     # embeddings (semantically meaningful once real weights are loaded);
@@ -194,7 +364,7 @@ class EngineConfig(BaseModel):
             return self.model
         return None
 
-    def resolve_arch(self) -> ModelArchConfig:
+    def resolve_arch(self):
         if self.model in MODEL_PRESETS:
             return MODEL_PRESETS[self.model]
         # A path: read config.json (HF-style) next to the weights
@@ -211,6 +381,11 @@ class EngineConfig(BaseModel):
             )
         with open(cfg_path) as f:
             hf = json.load(f)
+        if str(hf.get("architecture", "")).lower() == "zutalix":
+            from .weights import safetensors_shapes
+
+            return HybridArchConfig.from_checkpoint_config(
+                hf, safetensors_shapes(os.path.dirname(cfg_path)))
         arch = "mixtral" if "mixtral" in hf.get("model_type", "").lower() or hf.get("num_local_experts") else "llama"
         return ModelArchConfig(
             arch=arch,

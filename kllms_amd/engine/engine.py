@@ -105,6 +105,12 @@ class _DecodeBatchState:
         self.top_ks = torch.tensor([s.sampling.top_k for s in streams], dtype=torch.int32, device=dev)
         self.seeds = torch.tensor([s.seed for s in streams], dtype=torch.int64, device=dev)
         self.steps = torch.tensor([s.step for s in streams], dtype=torch.int64, device=dev)
+        # stateful models: every stream is a one-row segment with its own slot
+        self.state_slots = self.cu = self.token_seg = None
+        if engine.stateful:
+            self.state_slots = torch.tensor([s.seq.state_slot for s in streams], dtype=torch.int32, device=dev)
+            self.cu = torch.arange(len(streams) + 1, dtype=torch.int32, device=dev)
+            self.token_seg = torch.arange(len(streams), dtype=torch.int32, device=dev)
 
     def apply_bt_updates(self, updates: List[tuple]) -> None:
         need = max(j for _, j, _ in updates) + 1
@@ -184,16 +190,20 @@ class LLMEngine:
         self.eos_token_ids = frozenset(ids)
 
         self.model = self._build_model()
+        # models with recurrent state run segment batches against a
+        # HybridStateCache (block tables + state slots)
+        self.stateful = bool(getattr(self.model, "stateful", False))
         self.kv = self._build_kv_cache()
-        # cross-request shared-prefix KV reuse (kvcache.PrefixCache)
+        # cross-request shared-prefix KV reuse (kvcache.PrefixCache); off for
+        # stateful models: recurrent state cannot be rebuilt from cached blocks
         self.prefix_cache = None
-        if config.enable_prefix_caching:
+        if config.enable_prefix_caching and not self.stateful:
             from .kvcache import PrefixCache
 
             max_pfx = max(8, int(self.kv.num_blocks * config.prefix_cache_fraction))
             self.prefix_cache = PrefixCache(self.kv, max_pfx)
         self._graph_runner = None
-        if config.use_hip_graphs and self.device.type == "cuda":
+        if config.use_hip_graphs and self.device.type == "cuda" and not self.stateful:
             from .graph_runner import DecodeGraphRunner
 
             self._graph_runner = DecodeGraphRunner(self, config.hip_graph_batch_sizes)
@@ -219,11 +229,9 @@ class LLMEngine:
             return None
 
     def _build_model(self):
-        from ..models.llama import LlamaForCausalLM
-        from ..models.mixtral import MixtralForCausalLM
+        from ..models.registry import model_class
 
-        cls = MixtralForCausalLM if self.arch.arch == "mixtral" else LlamaForCausalLM
-        model = cls(self.arch, self.ctx, dtype=self.dtype)
+        model = model_class(self.arch.arch)(self.arch, self.ctx, dtype=self.dtype)
         wdir = self.config.effective_weights_dir()
         if wdir:
             from .weights import load_safetensors_weights
@@ -236,7 +244,36 @@ class LLMEngine:
         model.eval()
         return model
 
+    def _build_state_cache(self) -> PagedKVCache:
+        """Cache + state manager of a stateful model: per-layer paged K/V for
+        its attention layers and per-sequence slots for its recurrent ones.
+        The slot pool is sized first (one per stream plus fork headroom), the
+        block pool takes the rest of the memory budget."""
+        from .kvcache import HybridStateCache
+
+        cfg = self.config
+        specs = self.model.cache_layout()
+        elem = torch.tensor([], dtype=self.dtype).element_size()
+        bs = cfg.kv_block_size
+        num_slots = cfg.max_state_slots or (cfg.max_batch_size + 8)
+        if cfg.max_kv_blocks is not None:
+            num_blocks = cfg.max_kv_blocks
+        elif self.device.type == "cuda":
+            free, _total = torch.cuda.mem_get_info(self.device)
+            budget = int(free * cfg.kv_memory_fraction)
+            slot_bytes = HybridStateCache.bytes_per_slot(specs, elem)
+            num_slots = max(1, min(num_slots, (budget // 2) // max(1, slot_bytes)))
+            budget -= num_slots * slot_bytes
+            num_blocks = max(64, budget // max(1, HybridStateCache.bytes_per_block(specs, bs, elem)))
+            # no sequence can use more than max_seq_len tokens per slot
+            num_blocks = min(num_blocks, num_slots * ((cfg.max_seq_len + bs - 1) // bs) + 64)
+        else:
+            num_blocks = 512
+        return HybridStateCache(specs, bs, int(num_blocks), int(num_slots), self.device, self.dtype)
+
     def _build_kv_cache(self) -> PagedKVCache:
+        if self.stateful:
+            return self._build_state_cache()
         a = self.arch
         tp = self.ctx.world_size
         kv_heads_local = max(1, a.num_kv_heads // tp)
@@ -400,7 +437,14 @@ class LLMEngine:
             pack_rows.append(i)
 
         logits_by_req: List[Optional[torch.Tensor]] = [None] * len(requests)
-        if pack_rows:
+        if pack_rows and self.stateful:
+            segs = [(parent_seqs[i], 0, len(requests[i].prompt_ids)) for i in pack_rows]
+            batch = self._segment_batch(segs, all_slots)
+            input_ids = torch.tensor(all_ids, dtype=torch.long, device=dev)
+            packed_logits = self.model.forward_prefill(input_ids, batch)
+            for row, i in enumerate(pack_rows):
+                logits_by_req[i] = packed_logits[row]
+        elif pack_rows:
             batch = ForwardBatch(
                 mode="prefill",
                 positions=torch.tensor(all_pos, dtype=torch.long, device=dev),
@@ -543,6 +587,11 @@ class LLMEngine:
         of the final chunk (want_logits=True)."""
         dev = self.device
         ids = torch.tensor(prompt_ids[start:end], dtype=torch.long, device=dev)
+        if self.stateful:
+            slots_all = self.kv.prefill_slot_mapping(seq)
+            batch = self._segment_batch([(seq, start, end - start)], slots_all[start:end])
+            hidden = self.model.forward_hidden(ids, batch)
+            return self.model.compute_logits(hidden[-1:]) if want_logits else None
         pos = torch.arange(start, end, dtype=torch.long, device=dev)
         slots_all = self.kv.prefill_slot_mapping(seq)
         slots = torch.tensor(slots_all[start:end], dtype=torch.long, device=dev)
@@ -564,6 +613,95 @@ class LLMEngine:
         if want_logits:
             return self.model.compute_logits(hidden[-1:])
         return None
+
+    # --- segment steps -------------------------------------------------------
+    def _segment_batch(self, segs: List[Tuple[SequenceKV, int, int]], slots: List[int]) -> ForwardBatch:
+        """ForwardBatch in segment form. segs: (sequence, first position,
+        row count) per segment, rows packed in that order; slots: the flat
+        cache slot of every row. The sequences' block lists must already
+        cover the new rows."""
+        dev = self.device
+        pos: List[int] = []
+        tseg: List[int] = []
+        cu = [0]
+        for b, (_seq, start, n) in enumerate(segs):
+            pos.extend(range(start, start + n))
+            tseg.extend([b] * n)
+            cu.append(cu[-1] + n)
+        width = max(1, max(len(seq.blocks) for seq, _, _ in segs))
+        bt = torch.zeros((len(segs), width), dtype=torch.int32)
+        for b, (seq, _, _) in enumerate(segs):
+            if seq.blocks:
+                bt[b, : len(seq.blocks)] = torch.tensor(seq.blocks, dtype=torch.int32)
+        i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+        return ForwardBatch(
+            mode="segments",
+            positions=torch.tensor(pos, dtype=torch.long, device=dev),
+            slot_mapping=torch.tensor(slots, dtype=torch.long, device=dev),
+            kv_caches=self.kv.layer_caches(),
+            cu_seqlens=i32(cu),
+            block_tables=bt.to(dev),
+            context_lens=i32([start + n for _, start, n in segs]),
+            seg_start=i32([start for _, start, _ in segs]),
+            state_slots=i32([seq.state_slot for seq, _, _ in segs]),
+            token_seg=i32(tseg),
+        )
+
+    def open_sequence(self) -> SequenceKV:
+        """An empty sequence to be fed step by step through step_segments()."""
+        if self.stateful:
+            return self.kv.open_sequence()
+        return SequenceKV(blocks=[], num_tokens=0)
+
+    @torch.inference_mode()
+    def step_segments(self, entries: List[Tuple[SequenceKV, List[int], List[int]]]) -> Optional[torch.Tensor]:
+        """ONE forward over a mixed batch: each entry continues a sequence by
+        its next tokens (a prompt portion of any length, or a single decoded
+        token) from whatever cache and state earlier steps left. ``want``
+        lists, per entry, the indices among its new tokens whose logits are
+        needed. Returns fp32 logits [n_wanted, V] in entry order (None when
+        nothing is wanted). The step function under generation's prefill
+        slices and decode steps, exposed for replaying recorded schedules."""
+        dev = self.device
+        entries = [e for e in entries if len(e[1]) > 0]
+        if not entries:
+            return None
+        ids: List[int] = []
+        slots: List[int] = []
+        segs: List[Tuple[SequenceKV, int, int]] = []
+        want_rows: List[int] = []
+        for seq, toks, want in entries:
+            start = seq.num_tokens
+            slots.extend(self.kv.extend(seq, len(toks)))
+            want_rows.extend(len(ids) + w for w in want)
+            ids.extend(toks)
+            segs.append((seq, start, len(toks)))
+        input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
+        if self.stateful:
+            batch = self._segment_batch(segs, slots)
+        else:
+            # attention-only models: one decode-mode row per token, each row
+            # attending to its own sequence's cache up to its position
+            width = max(len(seq.blocks) for seq, _, _ in segs)
+            rows_bt = torch.zeros((len(ids), width), dtype=torch.int32)
+            pos: List[int] = []
+            r = 0
+            for seq, start, n in segs:
+                rows_bt[r : r + n, : len(seq.blocks)] = torch.tensor(seq.blocks, dtype=torch.int32)
+                pos.extend(range(start, start + n))
+                r += n
+            batch = ForwardBatch(
+                mode="decode",
+                positions=torch.tensor(pos, dtype=torch.long, device=dev),
+                slot_mapping=torch.tensor(slots, dtype=torch.long, device=dev),
+                kv_caches=self.kv.layer_caches(),
+                block_tables=rows_bt.to(dev),
+                context_lens=torch.tensor([p + 1 for p in pos], dtype=torch.int32, device=dev),
+            )
+        hidden = self.model.forward_hidden(input_ids, batch)
+        if not want_rows:
+            return None
+        return self.model.compute_logits(hidden[torch.tensor(want_rows, dtype=torch.long, device=dev)])
 
     def finish_stream(self, s: _Stream) -> StreamOutput:
         """Phase 3: detokenize (unless a stop-string already trimmed the
@@ -653,6 +791,11 @@ class LLMEngine:
             block_tables=state.bt,
             context_lens=state.ctx,
         )
+        if self.stateful:
+            batch.cu_seqlens = state.cu
+            batch.seg_start = state.positions.to(torch.int32)
+            batch.state_slots = state.state_slots
+            batch.token_seg = state.token_seg
         if self._graph_runner is not None:
             return self._graph_runner.run(state.ids, batch)
         return self.model.forward_decode(state.ids, batch)

@@ -64,6 +64,9 @@ class SequenceKV:
 
     blocks: List[int] = field(default_factory=list)
     num_tokens: int = 0
+    # recurrent-state slot (models with linear-attention / delta-rule /
+    # convolution state); -1 for pure-attention models
+    state_slot: int = -1
 
 
 class PagedKVCache:
@@ -169,6 +172,25 @@ class PagedKVCache:
         seq.num_tokens += 1
         return seq.blocks[blk_idx] * self.block_size + off
 
+    def extend(self, seq: SequenceKV, n_new: int) -> list[int]:
+        """Reserve room for n_new more tokens at the end of a sequence
+        (allocating blocks as needed) and return their flat slots. The
+        sequence's tail block must be private (not shared with a fork)."""
+        bs = self.block_size
+        start = seq.num_tokens
+        need = (start + n_new + bs - 1) // bs
+        added: List[int] = []
+        try:
+            while len(seq.blocks) + len(added) < need:
+                added.append(self.allocator.alloc())
+        except Exception:
+            for b in added:
+                self.allocator.free(b)
+            raise
+        seq.blocks.extend(added)
+        seq.num_tokens = start + n_new
+        return [seq.blocks[p // bs] * bs + p % bs for p in range(start, start + n_new)]
+
     def prefill_slot_mapping(self, seq: SequenceKV, start: int = 0) -> list[int]:
         """Flat slots for tokens [start, seq.num_tokens) of a fresh sequence."""
         slots = []
@@ -181,6 +203,150 @@ class PagedKVCache:
             self.allocator.free(b)
         seq.blocks = []
         seq.num_tokens = 0
+
+
+@dataclass
+class LayerCacheSpec:
+    """What one layer keeps between steps. kv = (kv_heads, key_dim, value_dim)
+    of a paged attention cache; rec = (heads, key_dim, value_dim) of an fp32
+    recurrent state matrix per head; conv = (channels, history) of carried
+    convolution inputs. None = the layer has no such state."""
+
+    kv: Optional[Tuple[int, int, int]] = None
+    rec: Optional[Tuple[int, int, int]] = None
+    conv: Optional[Tuple[int, int]] = None
+
+
+@dataclass
+class LayerState:
+    """One layer's device tensors: paged k/v [NB, G, BS, D|Dv], recurrent
+    state [slots, H, D, V] fp32, convolution history [slots, K-1, C]."""
+
+    k: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    rec: Optional[torch.Tensor] = None
+    conv: Optional[torch.Tensor] = None
+
+
+class StateSlotPool:
+    """Fixed pool of recurrent-state slots, one per live sequence. A slot is
+    not cleared when it changes hands: the kernels take the state of a
+    sequence's first step as zero whatever the slot holds."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free: List[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise RuntimeError("recurrent state out of slots")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        assert 0 <= slot < self.num_slots and slot not in self._free
+        self._free.append(slot)
+
+
+class HybridStateCache(PagedKVCache):
+    """Cache and state manager for models whose layers are listed one by one
+    and may each keep a paged attention cache, a recurrent state, a
+    convolution history, or several of these. Block ids are shared by all
+    attention layers (one block table per sequence), slots by all recurrent
+    layers; per-layer tensors may differ in head count and sizes.
+
+    Same sequence interface as PagedKVCache (alloc / extend / fork / free), so
+    the engine and scheduler drive both alike; fork copies the state slot the
+    way it copies a partially filled tail block."""
+
+    def __init__(self, specs: List[LayerCacheSpec], block_size: int, num_blocks: int, num_slots: int,
+                 device, dtype=torch.bfloat16):
+        self.num_layers = len(specs)
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.device = device
+        self.fp8 = False
+        self.specs = specs
+        self.layers: List[LayerState] = []
+        for sp in specs:
+            st = LayerState()
+            if sp.kv is not None:
+                g, d, dv = sp.kv
+                st.k = torch.zeros(num_blocks, g, block_size, d, device=device, dtype=dtype)
+                st.v = torch.zeros(num_blocks, g, block_size, dv, device=device, dtype=dtype)
+            if sp.rec is not None:
+                h, d, v = sp.rec
+                st.rec = torch.zeros(num_slots, h, d, v, device=device, dtype=torch.float32)
+            if sp.conv is not None:
+                c, hist = sp.conv
+                st.conv = torch.zeros(num_slots, hist, c, device=device, dtype=dtype)
+            self.layers.append(st)
+        self.allocator = BlockAllocator(num_blocks)
+        self.slots = StateSlotPool(num_slots)
+
+    @staticmethod
+    def bytes_per_block(specs: List[LayerCacheSpec], block_size: int, elem: int) -> int:
+        return sum(sp.kv[0] * block_size * (sp.kv[1] + sp.kv[2]) * elem for sp in specs if sp.kv)
+
+    @staticmethod
+    def bytes_per_slot(specs: List[LayerCacheSpec], elem: int) -> int:
+        n = 0
+        for sp in specs:
+            if sp.rec:
+                n += sp.rec[0] * sp.rec[1] * sp.rec[2] * 4
+            if sp.conv:
+                n += sp.conv[0] * sp.conv[1] * elem
+        return n
+
+    def layer_caches(self) -> List[LayerState]:
+        return self.layers
+
+    def _copy_block(self, src: int) -> int:
+        dst = self.allocator.alloc()
+        for st in self.layers:
+            if st.k is not None:
+                st.k[dst].copy_(st.k[src])
+                st.v[dst].copy_(st.v[src])
+        return dst
+
+    def open_sequence(self) -> SequenceKV:
+        """An empty sequence holding a state slot; grow it with extend()."""
+        return SequenceKV(blocks=[], num_tokens=0, state_slot=self.slots.alloc())
+
+    def alloc_sequence(self, num_tokens: int) -> SequenceKV:
+        slot = self.slots.alloc()
+        try:
+            seq = super().alloc_sequence(num_tokens)
+        except Exception:
+            self.slots.free(slot)
+            raise
+        seq.state_slot = slot
+        return seq
+
+    def fork(self, parent: SequenceKV) -> SequenceKV:
+        slot = self.slots.alloc()
+        try:
+            child = super().fork(parent)
+        except Exception:
+            self.slots.free(slot)
+            raise
+        child.state_slot = slot
+        if parent.state_slot >= 0:
+            for st in self.layers:
+                if st.rec is not None:
+                    st.rec[slot].copy_(st.rec[parent.state_slot])
+                if st.conv is not None:
+                    st.conv[slot].copy_(st.conv[parent.state_slot])
+        return child
+
+    def free_sequence(self, seq: SequenceKV) -> None:
+        super().free_sequence(seq)
+        if seq.state_slot >= 0:
+            self.slots.free(seq.state_slot)
+            seq.state_slot = -1
 
 
 class PrefixCache:

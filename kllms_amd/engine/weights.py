@@ -24,6 +24,23 @@ def _shard(t: torch.Tensor, dim: int, rank: int, world: int) -> torch.Tensor:
     return t.narrow(dim, rank * size, size)
 
 
+def safetensors_shapes(weights_dir: str) -> Dict[str, list]:
+    """Tensor name -> shape for every *.safetensors file in a directory, read
+    from the file headers only (8-byte little-endian length + JSON)."""
+    import json
+    import struct
+
+    out: Dict[str, list] = {}
+    for f in sorted(glob.glob(os.path.join(weights_dir, "*.safetensors"))):
+        with open(f, "rb") as fh:
+            (n,) = struct.unpack("<Q", fh.read(8))
+            header = json.loads(fh.read(n))
+        for name, meta in header.items():
+            if name != "__metadata__":
+                out[name] = list(meta["shape"])
+    return out
+
+
 @torch.no_grad()
 def load_safetensors_weights(model, weights_dir: str, ctx: ParallelContext) -> None:
     from safetensors import safe_open
@@ -32,6 +49,17 @@ def load_safetensors_weights(model, weights_dir: str, ctx: ParallelContext) -> N
     files = sorted(glob.glob(os.path.join(weights_dir, "*.safetensors")))
     if not files:
         raise FileNotFoundError(f"no .safetensors files under {weights_dir}")
+    if hasattr(model, "load_named_tensors_"):
+        # families whose checkpoint names are their own (listed-layer hybrids):
+        # the model maps names to its fused parameters itself
+        def stream():
+            for f in files:
+                with safe_open(f, framework="pt") as sf:
+                    for name in sf.keys():
+                        yield name, sf.get_tensor(name)
+
+        model.load_named_tensors_(stream())
+        return
 
     params: Dict[str, torch.Tensor] = dict(model.named_parameters())
     cfg = model.cfg

@@ -31,13 +31,21 @@ from ..parallel.tp import ColumnParallelLinear, ParallelContext, RowParallelLine
 
 @dataclass
 class ForwardBatch:
-    mode: Literal["prefill", "decode"]
+    mode: Literal["prefill", "decode", "segments"]
     positions: torch.Tensor              # [T] long
     slot_mapping: torch.Tensor           # [T] long — flat KV slots to write
     kv_caches: List[Tuple]  # per layer (k, v, k_scale|None, v_scale|None)
     cu_seqlens: Optional[torch.Tensor] = None   # [n_seq+1] int32 (prefill)
     block_tables: Optional[torch.Tensor] = None  # [B, max_blocks] int32 (decode)
     context_lens: Optional[torch.Tensor] = None  # [B] int32 (decode)
+    # segment form, used by models with recurrent state (any mix of prompt
+    # portions and single decoded tokens in one step): rows
+    # cu_seqlens[b]..cu_seqlens[b+1] continue sequence b at position
+    # seg_start[b]; block_tables has one row per SEGMENT; kv_caches holds one
+    # engine.kvcache.LayerState per layer
+    seg_start: Optional[torch.Tensor] = None     # [B] int32
+    state_slots: Optional[torch.Tensor] = None   # [B] int32
+    token_seg: Optional[torch.Tensor] = None     # [T] int32 — segment of each row
 
 
 class LlamaAttention(nn.Module):

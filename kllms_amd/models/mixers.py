@@ -1,0 +1,270 @@
+"""Sequence mixers and feed-forward blocks with their constants as
+parameters: block-local softmax attention over the paged cache, decayed
+linear attention, the gated delta rule with per-channel decay and short
+convolutions, and the clamped GLU. Each runs on "segment" batches
+(ForwardBatch.seg_start / state_slots / token_seg): any mix of prompt
+portions and single decoded tokens, attention keys found through the block
+table and recurrent state carried in per-sequence slots.
+
+GEMMs go through F.linear (hipBLASLt / rocBLAS); everything between them is a
+kllms_amd.ops kernel. Activations are the model dtype (bf16 when serving,
+fp32 in exact mode); norm weights, recurrence constants, attention weights
+and recurrent state are fp32 in both.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import ops
+from ..engine.config import (BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec,
+                             ParallelMixerSpec, RotarySpec)
+from ..engine.kvcache import LayerCacheSpec, LayerState
+
+
+def _param(*shape, dtype) -> nn.Parameter:
+    return nn.Parameter(torch.empty(*shape, dtype=dtype), requires_grad=False)
+
+
+def rotary_inv_freq(rot: RotarySpec) -> torch.Tensor:
+    """fp32 [dims/2] frequencies base^(-2i/dims), with the banded rescale:
+    wavelengths shorter than original/high keep their frequency, longer than
+    original/low are slowed by ``factor``, the band between blends the two
+    linearly in original/wavelength."""
+    n = rot.dims // 2
+    f = [float(rot.base) ** (-2.0 * i / rot.dims) for i in range(n)]
+    sc = rot.scaling
+    if sc:
+        fac, lo, hi, orig = (float(sc[k]) for k in ("factor", "low", "high", "original"))
+        out = []
+        for fi in f:
+            wl = 2.0 * math.pi / fi
+            if wl < orig / hi:
+                out.append(fi)
+            elif wl > orig / lo:
+                out.append(fi / fac)
+            else:
+                s = (orig / wl - lo) / (hi - lo)
+                out.append((1.0 - s) * fi / fac + s * fi)
+        f = out
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+
+
+class FusedInput(nn.Module):
+    """Several projections of the same input as ONE GEMM: the checkpoint's
+    separate [out_i, in] matrices are stacked along the output dim (optionally
+    with a bias that is zero where a part has none). ``parts`` keeps each
+    name's column range; ``split`` returns row views of the result."""
+
+    def __init__(self, in_features: int, parts: List[Tuple[str, int]], dtype, bias_parts=()):
+        super().__init__()
+        self.parts: Dict[str, Tuple[int, int]] = {}
+        off = 0
+        for name, n in parts:
+            self.parts[name] = (off, n)
+            off += n
+        self.weight = _param(off, in_features, dtype=dtype)
+        self.bias = _param(off, dtype=dtype) if bias_parts else None
+        self.bias_parts = tuple(bias_parts)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+    def split(self, y: torch.Tensor, name: str) -> torch.Tensor:
+        off, n = self.parts[name]
+        return y[:, off:off + n]
+
+    def slot(self, name: str) -> torch.Tensor:
+        off, n = self.parts[name]
+        return self.weight[off:off + n]
+
+    def bias_slot(self, name: str) -> torch.Tensor:
+        off, n = self.parts[name]
+        return self.bias[off:off + n]
+
+
+class BlockLocalAttention(nn.Module):
+    """GQA softmax attention whose causal mask is cut into aligned blocks of
+    ``mask_size`` positions (counted from the start of the sequence), rotary on
+    the first ``rot.dims`` dims (interleaved pairs), values optionally taken
+    from the un-rotated keys, per-head sigmoid output gate. Projections are
+    owned by the enclosing mixer (they share its fused input GEMM)."""
+
+    def __init__(self, spec: BlockAttnSpec, hidden: int, dtype):
+        super().__init__()
+        assert spec.heads % spec.kv_heads == 0
+        if spec.values_from_keys:
+            assert spec.vdim == spec.dim, "values taken from keys need vdim == dim"
+        self.spec = spec
+        self.o_proj = _param(hidden, spec.heads * spec.vdim, dtype=dtype)
+        self.register_buffer("inv_freq", rotary_inv_freq(spec.rot), persistent=False)
+
+    def cache_spec(self) -> Tuple[int, int, int]:
+        return (self.spec.kv_heads, self.spec.dim, self.spec.vdim)
+
+    def forward(self, q, k, v, gate, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        T = q.shape[0]
+        q = q.unflatten(1, (sp.heads, sp.dim))
+        k = k.unflatten(1, (sp.kv_heads, sp.dim))
+        if v is not None:
+            v = v.unflatten(1, (sp.kv_heads, sp.vdim))
+        ops.rope_pairs_store(q, k, v, batch.positions, self.inv_freq, st.k, st.v, batch.slot_mapping)
+        att = ops.attn_blocklocal_paged(q, st.k, st.v, batch.block_tables, batch.token_seg,
+                                        batch.positions, sp.scale, sp.mask_size, gate)
+        return F.linear(att.reshape(T, -1), self.o_proj)
+
+
+class DecayLinearAttention(nn.Module):
+    """S <- decay_h S + k v^T, o = S^T q with silu on q, k, v; the heads'
+    outputs are RMS-normed together, gated by sigmoid(g) and projected."""
+
+    def __init__(self, spec: DecayLinearAttnSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert len(spec.decay) == spec.heads
+        self.spec = spec
+        self.eps = eps
+        self.norm = _param(spec.heads * spec.vdim, dtype=torch.float32)
+        self.o_proj = _param(hidden, spec.heads * spec.vdim, dtype=dtype)
+        self.register_buffer("decay", torch.tensor(spec.decay, dtype=torch.float64).to(torch.float32),
+                             persistent=False)
+
+    def cache_spec(self) -> Tuple[int, int, int]:
+        return (self.spec.heads, self.spec.dim, self.spec.vdim)
+
+    def forward(self, q, k, v, gate, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        o = ops.linear_attn_decay(q.unflatten(1, (sp.heads, sp.dim)), k.unflatten(1, (sp.heads, sp.dim)),
+                                  v.unflatten(1, (sp.heads, sp.vdim)), self.decay, st.rec,
+                                  batch.state_slots, batch.cu_seqlens, batch.seg_start)
+        y = ops.gated_rmsnorm(o.view(o.shape[0], 1, -1), self.norm, gate, self.eps, self.o_proj.dtype)
+        return F.linear(y, self.o_proj)
+
+
+class ParallelMixer(nn.Module):
+    """Block-local softmax attention and decayed linear attention side by
+    side on the same input. Returns both branch outputs with their merge
+    weights; the caller's fused epilogue forms
+    (rms(left) w_left + rms(right) w_right) / 2."""
+
+    def __init__(self, spec: ParallelMixerSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        le, ri = spec.left, spec.right
+        parts = [("left.q", le.heads * le.dim), ("left.k", le.kv_heads * le.dim)]
+        if not le.values_from_keys:
+            parts.append(("left.v", le.kv_heads * le.vdim))
+        parts += [("right.q", ri.heads * ri.dim), ("right.k", ri.heads * ri.dim),
+                  ("right.v", ri.heads * ri.vdim), ("right.g", ri.heads * ri.vdim)]
+        if le.head_gate:
+            parts.append(("left.g", le.heads))          # odd-sized part last: the others stay aligned
+        self.inp = FusedInput(hidden, parts, dtype, bias_parts=("left.q", "left.k") if le.qk_bias else ())
+        self.left = BlockLocalAttention(le, hidden, dtype)
+        self.right = DecayLinearAttention(ri, hidden, eps, dtype)
+        self.left_out = _param(hidden, dtype=torch.float32)
+        self.right_out = _param(hidden, dtype=torch.float32)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        return LayerCacheSpec(kv=self.left.cache_spec(), rec=self.right.cache_spec())
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState):
+        y = self.inp(h)
+        s = self.inp.split
+        le = self.left.spec
+        left = self.left(s(y, "left.q"), s(y, "left.k"),
+                         None if le.values_from_keys else s(y, "left.v"),
+                         s(y, "left.g") if le.head_gate else None, batch, st)
+        right = self.right(s(y, "right.q"), s(y, "right.k"), s(y, "right.v"), s(y, "right.g"), batch, st)
+        return left, right
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        for n in self.inp.bias_parts:
+            m[pre + n + ".b"] = self.inp.bias_slot(n)
+        m[pre + "left.o"] = self.left.o_proj
+        m[pre + "right.o"] = self.right.o_proj
+        m[pre + "right.norm"] = self.right.norm
+        m[pre + "left.out"] = self.left_out
+        m[pre + "right.out"] = self.right_out
+        return m
+
+
+class ChannelDeltaMixer(nn.Module):
+    """Gated delta rule with one decay per head and key channel:
+        g = exp(-exp(A_h) softplus(W_a2 W_a1 h + dt));  S <- g (.) S
+        u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    q/k/v pass a short causal convolution + silu; q, k are unit-normalised;
+    each head's o is RMS-normed, gated by sigmoid(W_g2 W_g1 h) and projected."""
+
+    def __init__(self, spec: ChannelDeltaSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert spec.heads % spec.kv_heads == 0
+        self.spec = spec
+        self.eps = eps
+        self.gd, self.hv = spec.kv_heads * spec.dim, spec.heads * spec.vdim
+        self.inp = FusedInput(hidden, [("q", self.gd), ("k", self.gd), ("v", self.hv),
+                                       ("a1", spec.decay_rank), ("g1", spec.gate_rank), ("b", spec.heads)], dtype)
+        self.conv = _param(2 * self.gd + self.hv, spec.conv, dtype=torch.float32)
+        self.a2 = _param(spec.heads * spec.dim, spec.decay_rank, dtype=dtype)
+        self.g2 = _param(self.hv, spec.gate_rank, dtype=dtype)
+        self.dt_bias = _param(spec.heads * spec.dim, dtype=torch.float32)
+        self.A_log = _param(spec.heads, dtype=torch.float32)
+        self.norm = _param(spec.vdim, dtype=torch.float32)
+        self.o_proj = _param(hidden, self.hv, dtype=dtype)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(rec=(sp.heads, sp.dim, sp.vdim), conv=(2 * self.gd + self.hv, sp.conv - 1))
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        y = self.inp(h)
+        s = self.inp.split
+        c = 2 * self.gd + self.hv
+        qkv = ops.causal_conv_silu(y[:, :c], self.conv, st.conv, batch.state_slots, batch.cu_seqlens,
+                                   batch.seg_start, batch.token_seg)
+        a = F.linear(s(y, "a1"), self.a2)
+        gate = F.linear(s(y, "g1"), self.g2)
+        o = ops.gated_delta_rule(
+            qkv[:, :self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
+            qkv[:, self.gd:2 * self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
+            qkv[:, 2 * self.gd:].unflatten(1, (sp.heads, sp.vdim)),
+            s(y, "b"), a, self.dt_bias, self.A_log, st.rec, batch.state_slots, batch.cu_seqlens,
+            batch.seg_start)
+        r = ops.gated_rmsnorm(o, self.norm, gate, self.eps, self.o_proj.dtype)
+        return F.linear(r, self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        gd = self.gd
+        m[pre + "q.conv"] = self.conv[:gd]
+        m[pre + "k.conv"] = self.conv[gd:2 * gd]
+        m[pre + "v.conv"] = self.conv[2 * gd:]
+        for n in ("a2", "g2", "dt_bias", "A_log", "norm"):
+            m[pre + n] = getattr(self, n)
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class ClampedGLU(nn.Module):
+    """y = W_down [ g sigmoid(alpha g) (u + 1) ], g = min(W_gate h, limit),
+    u = clamp(W_up h, -limit, limit); gate and up share one GEMM."""
+
+    def __init__(self, spec: GluSpec, hidden: int, dtype):
+        super().__init__()
+        self.spec = spec
+        self.inp = FusedInput(hidden, [("gate", spec.ff), ("up", spec.ff)], dtype)
+        self.down = _param(hidden, spec.ff, dtype=dtype)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        y = self.inp(h)
+        act = ops.clamped_glu(self.inp.split(y, "gate"), self.inp.split(y, "up"),
+                              self.spec.limit, self.spec.alpha)
+        return F.linear(act, self.down)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        return {pre + "gate": self.inp.slot("gate"), pre + "up": self.inp.slot("up"), pre + "down": self.down}

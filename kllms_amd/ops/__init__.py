@@ -213,3 +213,123 @@ def levenshtein_pairs(
     normalized strings; returns int32 distances per (i, j) pair. GPU-only —
     the CPU consensus path keeps the pure-python DP (utils/text.py)."""
     return _hip_or_raise().levenshtein_pairs(chars, lens, pair_i, pair_j)
+
+
+# --- sequence-mixer family (kllms_amd._C_seq) -----------------------------------
+# fp32 residual stream, block-local paged attention, recurrent mixers. The
+# extension is separate from _C so that a model of this family compiles only
+# its own kernels in a checkout where nothing is built yet.
+
+_SEQ = None
+
+
+def _seq():
+    global _SEQ
+    if _SEQ is None:
+        from . import jit
+
+        _SEQ = jit.load("_C_seq")
+    return _SEQ
+
+
+def seq_hip_loaded() -> bool:
+    return _SEQ is not None
+
+
+def _gpu(t: torch.Tensor) -> bool:
+    return t.is_cuda and not _force_torch()
+
+
+def _none(ref: torch.Tensor, dtype=None) -> torch.Tensor:
+    return torch.empty(0, dtype=dtype or ref.dtype, device=ref.device)
+
+
+def embed_rmsnorm(ids, table, weight, eps):
+    if _gpu(table):
+        out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
+        _seq().embed_rmsnorm(out, ids, table, weight, eps)
+        return out
+    return torch_ref.embed_rmsnorm(ids, table, weight, eps)
+
+
+def rmsnorm_cast(x, weight, eps, out_dtype):
+    if _gpu(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _seq().rmsnorm_cast(out, x, weight, eps)
+        return out
+    return torch_ref.rmsnorm_cast(x, weight, eps, out_dtype)
+
+
+def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None):
+    """x (fp32 residual, in place) += rms(y) * w_post with y = a, or
+    y = (rms(a) wa + rms(b) wb) / 2; returns rms(x) * w_next in out_dtype
+    (None when w_next is None)."""
+    if _gpu(x):
+        out = torch.empty(a.shape, dtype=a.dtype, device=a.device) if w_next is not None else _none(a)
+        f = _none(x, torch.float32)
+        _seq().sandwich_residual(
+            x, a, b if b is not None else _none(a), wa if b is not None else f, wb if b is not None else f,
+            w_post, w_next if w_next is not None else f, out, eps)
+        return out if w_next is not None else None
+    return torch_ref.sandwich_residual(x, a, w_post, eps, b, wa, wb, w_next, out_dtype or a.dtype)
+
+
+def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping) -> None:
+    if _gpu(q):
+        _seq().rope_pairs_store(q, k, v if v is not None else _none(q), positions, inv_freq,
+                                k_cache, v_cache, slot_mapping)
+        return
+    torch_ref.rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping)
+
+
+def attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_size,
+                          gate=None):
+    if _gpu(q):
+        out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
+        _seq().attn_blocklocal_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions,
+                                     gate if gate is not None else _none(q), scale, mask_size)
+        return out
+    return torch_ref.attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions,
+                                           scale, mask_size, gate)
+
+
+def linear_attn_decay(q, k, v, decay, state, state_slots, cu_seqlens, seg_start):
+    if _gpu(q):
+        o = torch.empty((q.shape[0], q.shape[1], v.shape[2]), dtype=torch.float32, device=q.device)
+        _seq().linear_attn_decay(o, q, k, v, decay, state, state_slots, cu_seqlens, seg_start)
+        return o
+    return torch_ref.linear_attn_decay(q, k, v, decay, state, state_slots, cu_seqlens, seg_start)
+
+
+def gated_rmsnorm(o, weight, gate, eps, out_dtype):
+    if _gpu(o):
+        out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
+        _seq().gated_rmsnorm(out, o, weight, gate, eps)
+        return out
+    return torch_ref.gated_rmsnorm(o, weight, gate, eps, out_dtype)
+
+
+def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg):
+    if _gpu(x):
+        y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq().causal_conv_silu(y, x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg)
+        return y
+    return torch_ref.causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start)
+
+
+def gated_delta_rule(q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots, cu_seqlens, seg_start):
+    if _gpu(q):
+        o = torch.empty((v.shape[0], v.shape[1], v.shape[2]), dtype=torch.float32, device=q.device)
+        _seq().gated_delta_rule(o, q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots,
+                                cu_seqlens, seg_start)
+        return o
+    return torch_ref.gated_delta_rule(q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots,
+                                      cu_seqlens, seg_start)
+
+
+def clamped_glu(gate, up, limit: float, alpha: float):
+    if _gpu(gate):
+        out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+        _seq().clamped_glu(out, gate, up, limit, alpha)
+        return out
+    return torch_ref.clamped_glu(gate, up, limit, alpha)

@@ -1,0 +1,153 @@
+// Rotary (interleaved pairs, partial width) + paged K/V store, and block-local
+// softmax attention over the paged cache. One kernel serves prompt portions,
+// single decoded tokens and mixed batches: every query row finds its keys
+// through its segment's block table, so the result does not depend on how the
+// prompt was cut into steps.
+
+#include "seq_common.h"
+
+// grid (T, H + G), 64 threads. Heads 0..H-1 are query heads (rotated in place),
+// H..H+G-1 key heads: rotated copy -> k_cache, value row (v, or the un-rotated
+// key when v == nullptr) -> v_cache. angle = float(pos) * inv_freq[i], fp32.
+template <typename T>
+__global__ void rope_pairs_store_kernel(T* __restrict__ q, const T* __restrict__ k,
+                                        const T* __restrict__ v, const int64_t* __restrict__ positions,
+                                        const float* __restrict__ inv_freq, T* __restrict__ k_cache,
+                                        T* __restrict__ v_cache, const int64_t* __restrict__ slots,
+                                        int H, int G, int D, int Dv, int R, int BS,
+                                        int q_stride, int k_stride, int v_stride) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float pos = (float)positions[t];
+  if (h < H) {
+    T* row = q + (int64_t)t * q_stride + (int64_t)h * D;
+    for (int i = threadIdx.x; i < R; i += blockDim.x) {
+      float s, c;
+      sincosf(pos * inv_freq[i], &s, &c);
+      const float u = ldf(row + 2 * i), w = ldf(row + 2 * i + 1);
+      stf(row + 2 * i, u * c - w * s);
+      stf(row + 2 * i + 1, w * c + u * s);
+    }
+    return;
+  }
+  const int g = h - H;
+  const int64_t slot = slots[t];
+  const int64_t blk = slot / BS, off = slot % BS;
+  const T* krow = k + (int64_t)t * k_stride + (int64_t)g * D;
+  T* kc = k_cache + ((blk * G + g) * BS + off) * D;
+  T* vc = v_cache + ((blk * G + g) * BS + off) * Dv;
+  if (v != nullptr) {
+    const T* vrow = v + (int64_t)t * v_stride + (int64_t)g * Dv;
+    for (int i = threadIdx.x; i < Dv; i += blockDim.x) vc[i] = vrow[i];
+  } else {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) vc[i] = krow[i];
+  }
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    float s, c;
+    sincosf(pos * inv_freq[i], &s, &c);
+    const float u = ldf(krow + 2 * i), w = ldf(krow + 2 * i + 1);
+    stf(kc + 2 * i, u * c - w * s);
+    stf(kc + 2 * i + 1, w * c + u * s);
+  }
+  for (int i = 2 * R + threadIdx.x; i < D; i += blockDim.x) kc[i] = krow[i];
+}
+
+// grid (T, H), one wave per (query row, head). Keys lo..p, lo = the start of
+// p's aligned block of mask_size positions (0 when mask_size == 0), in tiles of
+// 64: lane j scores key lo + tile*64 + j (q staged in LDS), the tile's weights
+// go through LDS, then lanes own output dims and sweep the tile's value rows.
+// Online softmax in fp32. Optional per-head sigmoid gate on the output.
+#define ATTN_MAX_ACC 8   // Dv <= 512
+template <typename T>
+__global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __restrict__ q,
+                                             const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                             const int* __restrict__ block_tables,
+                                             const int* __restrict__ token_seg,
+                                             const int64_t* __restrict__ positions,
+                                             const T* __restrict__ gate, float scale, int mask_size,
+                                             int H, int G, int D, int Dv, int BS, int bt_stride,
+                                             int q_stride, int gate_stride) {
+  extern __shared__ float lds[];       // q [D] | p [64] | key row index [64] (as int)
+  float* qs = lds;
+  float* ps = lds + D;
+  int* rows = (int*)(ps + WAVE);
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (H / G);
+  const int p = (int)positions[t];
+  const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
+  const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
+  const T* qrow = q + (int64_t)t * q_stride + (int64_t)h * D;
+  for (int i = lane; i < D; i += WAVE) qs[i] = ldf(qrow + i) * scale;
+  __syncthreads();
+
+  float acc[ATTN_MAX_ACC];
+#pragma unroll
+  for (int i = 0; i < ATTN_MAX_ACC; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  for (int base = lo; base <= p; base += WAVE) {
+    const int j = base + lane;
+    float s = -INFINITY;
+    int row = -1;
+    if (j <= p) {
+      row = (bt[j / BS] * G + g) * BS + (j % BS);
+      const T* kr = k_cache + (int64_t)row * D;
+      float d = 0.f;
+      for (int i = 0; i < D; ++i) d += qs[i] * ldf(kr + i);
+      s = d;
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float w = j <= p ? expf(s - m_new) : 0.f;
+    const float corr = expf(m - m_new);        // m = -inf on the first tile -> 0
+    l = l * corr + wave_sum(w);
+    m = m_new;
+    ps[lane] = w;
+    rows[lane] = row;
+    __syncthreads();
+    const int n = min(WAVE, p - base + 1);
+#pragma unroll
+    for (int i = 0; i < ATTN_MAX_ACC; ++i) acc[i] *= corr;
+    for (int jj = 0; jj < n; ++jj) {
+      const float pw = ps[jj];
+      const T* vr = v_cache + (int64_t)rows[jj] * Dv;
+#pragma unroll
+      for (int i = 0; i < ATTN_MAX_ACC; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < Dv) acc[i] += pw * ldf(vr + d);
+      }
+    }
+    __syncthreads();
+  }
+  float gsc = 1.0f / l;
+  if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+  T* orow = out + ((int64_t)t * H + h) * Dv;
+#pragma unroll
+  for (int i = 0; i < ATTN_MAX_ACC; ++i) {
+    const int d = lane + i * WAVE;
+    if (d < Dv) stf(orow + d, acc[i] * gsc);
+  }
+}
+
+#define DISPATCH_T(is_f32, ...)                                  \
+  if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
+
+extern "C" void seq_launch_rope_pairs_store(void* q, const void* k, const void* v, const int64_t* positions,
+                                            const float* inv_freq, void* k_cache, void* v_cache,
+                                            const int64_t* slots, int T_, int H, int G, int D, int Dv, int R,
+                                            int BS, int q_stride, int k_stride, int v_stride, int is_f32,
+                                            hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(rope_pairs_store_kernel<T>, dim3(T_, H + G), dim3(WAVE), 0, st,
+                                        (T*)q, (const T*)k, (const T*)v, positions, inv_freq, (T*)k_cache,
+                                        (T*)v_cache, slots, H, G, D, Dv, R, BS, q_stride, k_stride, v_stride);)
+}
+
+extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const void* k_cache,
+                                                 const void* v_cache, const int* block_tables,
+                                                 const int* token_seg, const int64_t* positions,
+                                                 const void* gate, float scale, int mask_size, int T_, int H,
+                                                 int G, int D, int Dv, int BS, int bt_stride, int q_stride,
+                                                 int gate_stride, int is_f32, hipStream_t st) {
+  const size_t lds = (size_t)(D + 2 * WAVE) * sizeof(float);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(T_, H), dim3(WAVE), lds, st,
+                                        (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
+                                        block_tables, token_seg, positions, (const T*)gate, scale, mask_size,
+                                        H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
+}

@@ -262,3 +262,186 @@ def sample(
 
     logprobs = base_logprobs[torch.arange(B, device=logits.device), tokens]
     return tokens, logprobs
+
+
+# --- listed-layer hybrid family: fp32 residual stream, block-local attention,
+# --- recurrent mixers ---------------------------------------------------------
+#
+# Batch convention shared by these ops ("segments"): the step's tokens are
+# packed [T, ...]; segment b covers rows cu_seqlens[b]..cu_seqlens[b+1] and
+# continues sequence b at position seg_start[b] (0 = a fresh sequence, whose
+# recurrent state is taken as zero whatever its slot holds). A decode step is
+# the case of all segments having one row.
+
+def embed_rmsnorm(ids: torch.Tensor, table: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """fp32 residual stream: rmsnorm(table[ids]) * weight."""
+    x = table[ids].float()
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+
+
+def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -> torch.Tensor:
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+
+
+def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None):
+    """x (fp32, in place) += rmsnorm(y) * w_post, where y = a, or with a second
+    branch y = (rmsnorm(a) * wa + rmsnorm(b) * wb) / 2. Returns
+    rmsnorm(x) * w_next cast to out_dtype (the next sublayer's input), or None
+    when w_next is None."""
+    def n(t):
+        t = t.float()
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+
+    y = a.float()
+    if b is not None:
+        y = 0.5 * (n(a) * wa.float() + n(b) * wb.float())
+    x.add_(n(y) * w_post.float())
+    if w_next is None:
+        return None
+    return (n(x) * w_next.float()).to(out_dtype)
+
+
+def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping) -> None:
+    """Interleaved-pair rotary embedding on the first 2*len(inv_freq) dims of
+    q [T,H,D] and k [T,G,D] (q in place), angle = position * inv_freq in fp32;
+    the ROTATED k goes to k_cache and v (or, when v is None, the UN-rotated k)
+    to v_cache at the flat slots. Caches: [NB, G, BS, D]."""
+    R = inv_freq.numel()
+    ang = positions.to(torch.float32)[:, None] * inv_freq.float()[None, :]   # [T, R]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+    def rot(t):
+        tf = t.float()
+        u, w = tf[..., 0:2 * R:2], tf[..., 1:2 * R:2]
+        out = tf.clone()
+        out[..., 0:2 * R:2] = u * cos - w * sin
+        out[..., 1:2 * R:2] = w * cos + u * sin
+        return out
+
+    BS = k_cache.shape[2]
+    blk, off = slot_mapping // BS, slot_mapping % BS
+    vals = k if v is None else v
+    v_cache[blk, :, off, :] = vals.to(v_cache.dtype)
+    k_cache[blk, :, off, :] = rot(k).to(k_cache.dtype)
+    q.copy_(rot(q).to(q.dtype))
+
+
+def attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale,
+                          mask_size, gate=None, out_dtype=None) -> torch.Tensor:
+    """Softmax attention of packed query rows against the paged cache. Row t
+    (segment token_seg[t], position p) sees keys lo..p of its own sequence,
+    lo = floor(p / mask_size) * mask_size (0 when mask_size == 0). ``gate``
+    [T, H] (logits): each head's output is scaled by its sigmoid."""
+    T, H, D = q.shape
+    _, G, BS, Dv = v_cache.shape
+    rep = H // G
+    out = torch.empty(T, H, Dv, dtype=out_dtype or q.dtype, device=q.device)
+    pos = positions.tolist()
+    seg = token_seg.tolist()
+    for t in range(T):
+        p = pos[t]
+        lo = (p // mask_size) * mask_size if mask_size > 0 else 0
+        idx = torch.arange(lo, p + 1, device=q.device)
+        blocks = block_tables[seg[t]].long()[idx // BS]
+        kk = k_cache[blocks, :, idx % BS, :].float()          # [n, G, D]
+        vv = v_cache[blocks, :, idx % BS, :].float()
+        qt = q[t].float().view(G, rep, D)
+        s = torch.einsum("grd,ngd->grn", qt, kk) * scale
+        pr = torch.softmax(s, dim=-1)
+        o = torch.einsum("grn,ngd->grd", pr, vv).reshape(H, Dv)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float())[:, None]
+        out[t] = o.to(out.dtype)
+    return out
+
+
+def linear_attn_decay(q, k, v, decay, state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
+    """Decayed linear attention over segments. q,k [T,H,D], v [T,H,V] are the
+    raw projections (silu is applied here); decay [H] fp32;
+    state [slots,H,D,V] fp32 is read (unless seg_start == 0) and written back.
+    Returns o [T,H,V] fp32 with o_t = S_t^T q_t, S_t = decay S_{t-1} + k_t v_t^T."""
+    T, H, _ = q.shape
+    qf = torch.nn.functional.silu(q.float())
+    kf = torch.nn.functional.silu(k.float())
+    vf = torch.nn.functional.silu(v.float())
+    o = torch.empty(T, H, v.shape[-1], dtype=torch.float32, device=q.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    d = decay.float().view(H, 1, 1)
+    for b in range(len(sl)):
+        S = state[sl[b]].clone() if st[b] > 0 else torch.zeros_like(state[sl[b]])
+        for t in range(cu[b], cu[b + 1]):
+            S = d * S + kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[sl[b]] = S
+    return o
+
+
+def gated_rmsnorm(o, weight, gate, eps, out_dtype) -> torch.Tensor:
+    """o [T, n_groups, S] fp32: each group is divided by its root mean square,
+    times weight [S], times sigmoid(gate) ([T, n_groups*S] logits).
+    Returns [T, n_groups*S]."""
+    T, Gn, S = o.shape
+    of = o.float()
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return (y.reshape(T, Gn * S) * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
+    """Per-channel causal convolution over time + silu. x [T,C]; w [C,K] (last
+    column = current token); conv_state [slots, K-1, C] holds each sequence's
+    last K-1 inputs (oldest first) and is updated."""
+    T, C = x.shape
+    K = w.shape[1]
+    y = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    wf = w.float()
+    for b in range(len(sl)):
+        s, e = cu[b], cu[b + 1]
+        hist = conv_state[sl[b]].float() if st[b] > 0 else torch.zeros(K - 1, C, device=x.device)
+        ext = torch.cat([hist, x[s:e].float()], 0)           # [K-1+L, C]
+        acc = torch.zeros(e - s, C, device=x.device)
+        for j in range(K):
+            acc += ext[j:j + (e - s)] * wf[:, j]
+        y[s:e] = torch.nn.functional.silu(acc).to(x.dtype)
+        conv_state[sl[b]] = ext[ext.shape[0] - (K - 1):].to(conv_state.dtype)
+    return y
+
+
+def gated_delta_rule(q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots, cu_seqlens,
+                     seg_start) -> torch.Tensor:
+    """Gated delta rule with a decay per head and key channel.
+    q,k [T,G,D], v [T,H,V] (already convolved + silu); beta_logit [T,H];
+    a [T,H*D] decay pre-activation (dt_bias [H*D] added here); a_log [H];
+    state [slots,H,D,V] fp32. Per head: S <- g*S (rows), u = beta (v - S^T k),
+    S <- S + k u^T, o = S^T q. q,k are unit-normalized (eps 1e-6 inside the
+    root) and q scaled by D^-1/2. Returns o [T,H,V] fp32."""
+    T, G, D = q.shape
+    H, V = v.shape[1], v.shape[2]
+    rep = H // G
+    qf, kf, vf = q.float(), k.float(), v.float()
+    qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + 1e-6) * (D ** -0.5)
+    kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qf = qf.repeat_interleave(rep, dim=1)
+    kf = kf.repeat_interleave(rep, dim=1)
+    beta = torch.sigmoid(beta_logit.float())
+    sp = torch.nn.functional.softplus(a.float() + dt_bias.float()).view(T, H, D)
+    g = torch.exp(-torch.exp(a_log.float()).view(1, H, 1) * sp)
+    o = torch.empty(T, H, V, dtype=torch.float32, device=q.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    for b in range(len(sl)):
+        S = state[sl[b]].clone() if st[b] > 0 else torch.zeros_like(state[sl[b]])
+        for t in range(cu[b], cu[b + 1]):
+            S = S * g[t].unsqueeze(-1)
+            pred = torch.einsum("hdv,hd->hv", S, kf[t])
+            u = beta[t].unsqueeze(-1) * (vf[t] - pred)
+            S = S + kf[t].unsqueeze(-1) * u.unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[sl[b]] = S
+    return o
+
+
+def clamped_glu(gate, up, limit: float, alpha: float) -> torch.Tensor:
+    g = gate.float().clamp(max=limit)
+    u = up.float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate.dtype)

@@ -3,10 +3,13 @@
     PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace
 
 Produces kllms_amd/_C*.so next to the package sources so the snapshot that
-ships to a GPU box carries the built extension.
+ships to a GPU box carries the built extension, then compiles the
+per-family extensions (kllms_amd/ops/jit.py: _C_seq) the same way they are
+compiled on demand in a checkout with nothing built.
 """
 
 import os
+import sys
 
 from setuptools import setup
 
@@ -38,9 +41,20 @@ setup(
             sources=SOURCES,
             extra_compile_args={
                 "cxx": ["-O3"],
-                "nvcc": ["-O3", "--offload-arch=gfx950", "-std=c++17"],
+                # packed-fp32 instruction selection is switched off for all
+                # device code (the host pass warns that it does not know the
+                # feature; harmless)
+                "nvcc": ["-O3", "--offload-arch=gfx950", "-std=c++17",
+                         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"],
             },
         )
     ],
     cmdclass={"build_ext": BuildExtension},
 )
+
+if "build_ext" in sys.argv:
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from kllms_amd.ops import jit
+
+    for _name in jit.EXTENSIONS:
+        print("built", jit.build(_name))
