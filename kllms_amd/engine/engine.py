@@ -203,7 +203,7 @@ class LLMEngine:
             max_pfx = max(8, int(self.kv.num_blocks * config.prefix_cache_fraction))
             self.prefix_cache = PrefixCache(self.kv, max_pfx)
         self._graph_runner = None
-        if config.use_hip_graphs and self.device.type == "cuda" and not self.stateful:
+        if config.use_hip_graphs and self.device.type == "cuda":
             from .graph_runner import DecodeGraphRunner
 
             self._graph_runner = DecodeGraphRunner(self, config.hip_graph_batch_sizes)

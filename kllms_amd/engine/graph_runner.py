@@ -32,6 +32,9 @@ class DecodeGraphRunner:
         self.max_blocks_per_seq = (engine.config.max_seq_len + engine.config.kv_block_size - 1) // engine.config.kv_block_size
         # one scratch block for padded lanes' KV writes
         self._scratch_block = engine.kv.allocator.alloc()
+        # stateful models: padded lanes run as fresh one-row segments whose
+        # recurrent state lands in a slot of their own
+        self._scratch_slot = engine.kv.slots.alloc() if engine.stateful else -1
         self._enabled = True
 
     def _capture(self, bs: int) -> None:
@@ -53,6 +56,13 @@ class DecodeGraphRunner:
             block_tables=buf["block_tables"],
             context_lens=buf["context_lens"],
         )
+        if eng.stateful:
+            buf["seg_start"] = torch.zeros(bs, dtype=torch.int32, device=dev)
+            buf["state_slots"] = torch.full((bs,), self._scratch_slot, dtype=torch.int32, device=dev)
+            batch.seg_start = buf["seg_start"]
+            batch.state_slots = buf["state_slots"]
+            batch.cu_seqlens = torch.arange(bs + 1, dtype=torch.int32, device=dev)
+            batch.token_seg = torch.arange(bs, dtype=torch.int32, device=dev)
         # warmup on a side stream (required before capture)
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -133,5 +143,10 @@ class DecodeGraphRunner:
         buf["block_tables"][B:].fill_(self._scratch_block)
         buf["context_lens"][:B].copy_(batch.context_lens)
         buf["context_lens"][B:].fill_(1)
+        if self.engine.stateful:
+            buf["seg_start"][:B].copy_(batch.seg_start)
+            buf["seg_start"][B:].fill_(0)
+            buf["state_slots"][:B].copy_(batch.state_slots)
+            buf["state_slots"][B:].fill_(self._scratch_slot)
         self.graphs[bs].replay()
         return self.engine.model.compute_logits(buf["out"][:B])

@@ -52,16 +52,26 @@ class ByteTokenizer(BaseTokenizer):
     N_BYTES = 256
 
     def __init__(self, vocab_size: int = 128256):
-        assert vocab_size >= self.N_BYTES + 3
         self.vocab_size = vocab_size
-        self.bos_id = self.N_BYTES
-        self.eos_id = self.N_BYTES + 1
-        self.pad_id = self.N_BYTES + 2
+        if vocab_size >= self.N_BYTES + 3:
+            self.bos_id = self.N_BYTES
+            self.eos_id = self.N_BYTES + 1
+            self.pad_id = self.N_BYTES + 2
+        else:
+            # toy vocabularies (tests, synthetic checkpoints): bytes fold
+            # into the ids there are and no id is reserved — generation ends
+            # by length only (eos -1 is never sampled)
+            self.N_BYTES = max(1, vocab_size)
+            self.bos_id = None
+            self.eos_id = -1
+            self.pad_id = 0
         self.cache_key = ("byte", vocab_size)
 
     def encode(self, text: str, add_bos: bool = False) -> list[int]:
         ids = list(text.encode("utf-8", errors="replace"))
-        if add_bos:
+        if self.N_BYTES < 256:
+            ids = [i % self.N_BYTES for i in ids]
+        if add_bos and self.bos_id is not None:
             ids = [self.bos_id] + ids
         return ids
 
