@@ -27,6 +27,12 @@ aggregate. ``--parallel tp`` instead shards ONE engine across all ranks
 (column/row-parallel layers + RCCL/xGMI all-reduce): rank 0 runs the client
 and scheduler, other ranks follow in lockstep (parallel/serve.py).
 
+``--compare-families`` is a separate, single-GPU measurement: prefill and
+decode token throughput of the Zutalix family (listed-layer hybrid) beside
+the dense Llama stack of the same width / depth / heads / ff, straight through
+LLMEngine.generate (random-init weights, synthetic token ids). It prints its
+own JSON line and leaves the default workload untouched.
+
 Usage: python bench.py [--gpus N] [--steps K] [--warmup W]
 Rank 0 prints exactly one JSON result line.
 """
@@ -152,8 +158,58 @@ CONFIG_DEFAULTS = {
 }
 
 
+def compare_families(args) -> None:
+    """Prefill / decode tokens per second of the two families at equal layer
+    shapes. One engine at a time; W warmup + K timed generate() calls each."""
+    from kllms_amd.engine.config import MODEL_PRESETS, EngineConfig
+    from kllms_amd.engine.engine import GenRequest, LLMEngine
+    from kllms_amd.engine.sampling import SamplingParams
+
+    device = "cuda:0" if torch.cuda.is_available() else "cpu"
+    sizes = [s for s in args.sizes.split(",") if s]
+    B, P, N = args.batch or 16, args.prompt_len, args.max_new or 64
+    rows = []
+    for size in sizes:
+        for fam in ("llama", "zutalix"):
+            name = f"{fam}-{size}" if f"{fam}-{size}" in MODEL_PRESETS else f"{size}-{fam}"
+            kw = dict(model=name, device=device, seed=0, use_hip_graphs=device != "cpu" and not args.no_graphs,
+                      max_seq_len=P + N + 64, max_batch_size=max(B, 8), enable_prefix_caching=False,
+                      eos_token_id=-1)     # no stop id: every stream decodes its N tokens
+            if device == "cpu":
+                kw["max_kv_blocks"] = 4096
+            eng = LLMEngine(EngineConfig(**kw))
+            g = torch.Generator().manual_seed(1)
+            mk = lambda: [GenRequest(prompt_ids=torch.randint(3, 250, (P,), generator=g).tolist(), n=1,
+                                     sampling=SamplingParams(temperature=1.0, max_tokens=N, seed=i))
+                          for i in range(B)]
+            pre = dec = 0.0
+            steps = 0
+            for it in range(args.warmup + args.steps):
+                eng.generate(mk())
+                if it >= args.warmup:
+                    t = eng.last_timings
+                    pre += t["prefill_ms"]
+                    dec += t["decode_ms"]
+                    steps += t["decode_steps"]
+            row = {"model": name, "batch": B, "prompt_len": P,
+                   "prefill_tok_s": round(B * P * args.steps / (pre / 1e3), 1),
+                   "decode_tok_s": round(B * steps / (dec / 1e3), 1),
+                   "prefill_ms": round(pre / args.steps, 2),
+                   "decode_ms_per_step": round(dec / max(1, steps), 3)}
+            log(f"[compare] {row}")
+            rows.append(row)
+            del eng
+            if device != "cpu":
+                torch.cuda.empty_cache()
+    print(json.dumps({"metric": "family_compare_tokens_per_s", "unit": "tok/s", "dtype": "bf16" if device != "cpu" else "fp32",
+                      "data": "synthetic", "steps": args.steps, "warmup": args.warmup, "rows": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--compare-families", action="store_true",
+                    help="prefill/decode tok/s of the Zutalix family beside the dense Llama stack of equal shape")
+    ap.add_argument("--sizes", type=str, default="1b-l6,8b-l6", help="--compare-families: preset size suffixes")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
@@ -167,6 +223,9 @@ def main():
     ap.add_argument("--parallel", type=str, default="dp", choices=["dp", "tp"],
                     help="dp: one engine per rank (weak scaling); tp: ONE engine sharded over all ranks")
     args = ap.parse_args()
+    if args.compare_families:
+        compare_families(args)
+        return
 
     cfgd = CONFIG_DEFAULTS[args.config]
     model = args.model or cfgd["model"]

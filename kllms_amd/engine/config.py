@@ -276,10 +276,21 @@ MODEL_PRESETS: dict = {
     "mid-zutalix": _zutalix_preset(
         vocab=2048, width=512, n_par=3, heads=4, kv_heads=2, dim=128, mask=256,
         lin_heads=4, lin_dim=64, lin_vdim=128, d_heads=4, d_kv=2, d_dim=64, d_vdim=128, ff=1024),
-    # layer shapes of an 8B-class model at reduced depth (bench sizes)
+    # layer shapes of real models at reduced depth, and the dense Llama stack
+    # of the same width / depth / heads / ff beside each (bench.py
+    # --compare-families)
     "zutalix-8b-l6": _zutalix_preset(
-        vocab=128256, width=4096, n_par=6, heads=32, kv_heads=8, dim=128, mask=2048,
+        vocab=32000, width=4096, n_par=6, heads=32, kv_heads=8, dim=128, mask=2048,
         lin_heads=32, lin_dim=128, lin_vdim=128, d_heads=32, d_kv=16, d_dim=128, d_vdim=128, ff=14336),
+    "llama-8b-l6": ModelArchConfig(
+        arch="llama", vocab_size=32000, hidden_size=4096, intermediate_size=14336,
+        num_layers=6, num_heads=32, num_kv_heads=8, rope_theta=500000.0),
+    "zutalix-1b-l6": _zutalix_preset(
+        vocab=32000, width=2048, n_par=6, heads=16, kv_heads=4, dim=128, mask=1024,
+        lin_heads=16, lin_dim=64, lin_vdim=128, d_heads=16, d_kv=8, d_dim=64, d_vdim=128, ff=8192),
+    "llama-1b-l6": ModelArchConfig(
+        arch="llama", vocab_size=32000, hidden_size=2048, intermediate_size=8192,
+        num_layers=6, num_heads=16, num_kv_heads=4, rope_theta=500000.0),
 }
 
 
