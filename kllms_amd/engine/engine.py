@@ -203,7 +203,15 @@ class LLMEngine:
             max_pfx = max(8, int(self.kv.num_blocks * config.prefix_cache_fraction))
             self.prefix_cache = PrefixCache(self.kv, max_pfx)
         self._graph_runner = None
-        if config.use_hip_graphs and self.device.type == "cuda":
+        if config.use_hip_graphs and self.device.type == "cuda" and self.stateful:
+            # capture of the stateful decode step is switched off: the one
+            # captured run of it aborted in graph teardown on hardware and the
+            # cause is not established; decode runs eagerly until it is
+            import logging
+
+            logging.getLogger("kllms_amd.engine").warning(
+                "decode graphs are off for models with recurrent state; running decode eagerly")
+        elif config.use_hip_graphs and self.device.type == "cuda":
             from .graph_runner import DecodeGraphRunner
 
             self._graph_runner = DecodeGraphRunner(self, config.hip_graph_batch_sizes)
