@@ -653,6 +653,8 @@ class LLMEngine:
             seg_start=i32([start for _, start, _ in segs]),
             state_slots=i32([seq.state_slot for seq, _, _ in segs]),
             token_seg=i32(tseg),
+            host_segs=[(start, n) for _, start, n in segs],
+            plans={},
         )
 
     def open_sequence(self) -> SequenceKV:

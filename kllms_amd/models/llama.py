@@ -46,6 +46,11 @@ class ForwardBatch:
     seg_start: Optional[torch.Tensor] = None     # [B] int32
     state_slots: Optional[torch.Tensor] = None   # [B] int32
     token_seg: Optional[torch.Tensor] = None     # [T] int32 — segment of each row
+    # host copy of (first position, row count) per segment, when the step was
+    # built on the host (absent for device-resident decode state): lets a
+    # layer plan per-piece kernels without a device sync; plans are cached here
+    host_segs: Optional[list] = None
+    plans: Optional[dict] = None
 
 
 class LlamaAttention(nn.Module):

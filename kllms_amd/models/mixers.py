@@ -107,6 +107,49 @@ class BlockLocalAttention(nn.Module):
     def cache_spec(self) -> Tuple[int, int, int]:
         return (self.spec.kv_heads, self.spec.dim, self.spec.vdim)
 
+    # pieces shorter than this stay on the paged kernel
+    MIN_DENSE_ROWS = 32
+
+    def _dense_plan(self, q: torch.Tensor, batch):
+        """Split the step's rows between the dense MFMA prefill kernel and the
+        paged kernel. A run of rows whose whole visible block lies inside this
+        step (it starts at a block boundary of the mask, or at position 0 for
+        a plain causal mask) is a 'piece': plain causal attention over fresh
+        rows. Rows that continue a block begun in an earlier step, and short
+        pieces, read their keys through the block table instead. Returns
+        (tile groups, row_map or None), or None when nothing goes dense."""
+        sp = self.spec
+        if (batch.host_segs is None or not q.is_cuda or q.dtype != torch.bfloat16
+                or sp.dim != 128 or sp.vdim != 128 or ops._force_torch()):
+            return None
+        key = ("blocklocal", sp.mask_size)
+        if key in batch.plans:
+            return batch.plans[key]
+        M = sp.mask_size
+        pieces, paged = [], []
+        row0 = 0
+        for start, n in batch.host_segs:
+            r = 0
+            if M > 0 and start % M:
+                r = min(n, M - start % M)
+            elif M == 0 and start > 0:
+                r = n
+            paged.extend(range(row0, row0 + r))
+            while r < n:
+                L = min(M, n - r) if M > 0 else n - r
+                if L >= self.MIN_DENSE_ROWS:
+                    pieces.append((row0 + r, L))
+                else:
+                    paged.extend(range(row0 + r, row0 + r + L))
+                r += L
+            row0 += n
+        plan = None
+        if pieces:
+            row_map = torch.tensor(paged, dtype=torch.int32, device=q.device) if paged else None
+            plan = (ops.dense_tile_groups(pieces, q.device), row_map)
+        batch.plans[key] = plan
+        return plan
+
     def forward(self, q, k, v, gate, batch, st: LayerState) -> torch.Tensor:
         sp = self.spec
         T = q.shape[0]
@@ -114,9 +157,23 @@ class BlockLocalAttention(nn.Module):
         k = k.unflatten(1, (sp.kv_heads, sp.dim))
         if v is not None:
             v = v.unflatten(1, (sp.kv_heads, sp.vdim))
-        ops.rope_pairs_store(q, k, v, batch.positions, self.inv_freq, st.k, st.v, batch.slot_mapping)
-        att = ops.attn_blocklocal_paged(q, st.k, st.v, batch.block_tables, batch.token_seg,
-                                        batch.positions, sp.scale, sp.mask_size, gate)
+        plan = self._dense_plan(q, batch)
+        if plan is None:
+            ops.rope_pairs_store(q, k, v, batch.positions, self.inv_freq, st.k, st.v, batch.slot_mapping)
+            att = ops.attn_blocklocal_paged(q, st.k, st.v, batch.block_tables, batch.token_seg,
+                                            batch.positions, sp.scale, sp.mask_size, gate)
+        else:
+            (gs, gq, gl), row_map = plan
+            fresh = torch.empty((T, 2, sp.kv_heads, sp.dim), dtype=q.dtype, device=q.device)
+            ops.rope_pairs_store(q, k, v, batch.positions, self.inv_freq, st.k, st.v, batch.slot_mapping,
+                                 kv_fresh=fresh)
+            att = torch.empty((T, sp.heads, sp.vdim), dtype=q.dtype, device=q.device)
+            ops.attn_varlen_mfma(att, q, fresh[:, 0], fresh[:, 1], gs, gq, gl, sp.scale)
+            if row_map is not None:
+                ops.attn_blocklocal_paged(q, st.k, st.v, batch.block_tables, batch.token_seg, batch.positions,
+                                          sp.scale, sp.mask_size, None, row_map=row_map, out=att)
+            if gate is not None:
+                ops.head_gate(att, gate)
         return F.linear(att.reshape(T, -1), self.o_proj)
 
 

@@ -274,23 +274,63 @@ def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, 
     return torch_ref.sandwich_residual(x, a, w_post, eps, b, wa, wb, w_next, out_dtype or a.dtype)
 
 
-def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping) -> None:
+def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping, kv_fresh=None) -> None:
+    """kv_fresh (GPU only, optional): [T, 2, G, D] buffer that also receives
+    this step's rotated keys ([:, 0]) and values ([:, 1]) packed, for the
+    dense prefill kernel."""
     if _gpu(q):
         _seq().rope_pairs_store(q, k, v if v is not None else _none(q), positions, inv_freq,
-                                k_cache, v_cache, slot_mapping)
+                                k_cache, v_cache, slot_mapping,
+                                kv_fresh if kv_fresh is not None else _none(q))
         return
     torch_ref.rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping)
 
 
 def attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_size,
-                          gate=None):
+                          gate=None, row_map=None, out=None):
+    """row_map / out (GPU only): serve just the listed rows, writing into an
+    existing [T, H, Dv] tensor whose other rows another kernel fills."""
     if _gpu(q):
-        out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
+        if out is None:
+            out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
         _seq().attn_blocklocal_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions,
-                                     gate if gate is not None else _none(q), scale, mask_size)
+                                     gate if gate is not None else _none(q), scale, mask_size,
+                                     row_map if row_map is not None else _none(q, torch.int32))
         return out
+    assert row_map is None and out is None
     return torch_ref.attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions,
                                            scale, mask_size, gate)
+
+
+def attn_varlen_mfma(out, q, k, v, grp_start, grp_qpos0, grp_len, scale) -> None:
+    """Dense causal MFMA attention over packed pieces (bf16, head size 128;
+    GPU only): each piece attends within itself. Tile groups come from
+    dense_tile_groups()."""
+    _seq().attn_varlen_mfma(out, q, k, v, grp_start, grp_qpos0, grp_len, scale)
+
+
+def dense_tile_groups(pieces, device):
+    """Host metadata for attn_varlen_mfma: pieces = [(first row, length)];
+    32-row q-tiles of each piece, 8 per workgroup (idle wave slots = -1)."""
+    NW = 8
+    gs, gl, gq = [], [], []
+    for row0, L in pieces:
+        tiles = list(range(0, L, 32))
+        for g0 in range(0, len(tiles), NW):
+            grp = tiles[g0:g0 + NW]
+            gs.append(row0)
+            gl.append(L)
+            gq.extend(grp + [-1] * (NW - len(grp)))
+    t = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    return t(gs), t(gq), t(gl)
+
+
+def head_gate(out, gate) -> None:
+    """out[t, h, :] *= sigmoid(gate[t, h]) in place."""
+    if _gpu(out):
+        _seq().head_gate(out, gate)
+        return
+    out.mul_(torch.sigmoid(gate.float()).unsqueeze(-1).to(out.dtype))
 
 
 def linear_attn_decay(q, k, v, decay, state, state_slots, cu_seqlens, seg_start):

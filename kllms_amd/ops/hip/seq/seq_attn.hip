@@ -14,7 +14,7 @@ __global__ void rope_pairs_store_kernel(T* __restrict__ q, const T* __restrict__
                                         const T* __restrict__ v, const int64_t* __restrict__ positions,
                                         const float* __restrict__ inv_freq, T* __restrict__ k_cache,
                                         T* __restrict__ v_cache, const int64_t* __restrict__ slots,
-                                        int H, int G, int D, int Dv, int R, int BS,
+                                        T* __restrict__ kv_fresh, int H, int G, int D, int Dv, int R, int BS,
                                         int q_stride, int k_stride, int v_stride) {
   const int t = blockIdx.x, h = blockIdx.y;
   const float pos = (float)positions[t];
@@ -35,11 +35,14 @@ __global__ void rope_pairs_store_kernel(T* __restrict__ q, const T* __restrict__
   const T* krow = k + (int64_t)t * k_stride + (int64_t)g * D;
   T* kc = k_cache + ((blk * G + g) * BS + off) * D;
   T* vc = v_cache + ((blk * G + g) * BS + off) * Dv;
-  if (v != nullptr) {
-    const T* vrow = v + (int64_t)t * v_stride + (int64_t)g * Dv;
-    for (int i = threadIdx.x; i < Dv; i += blockDim.x) vc[i] = vrow[i];
-  } else {
-    for (int i = threadIdx.x; i < D; i += blockDim.x) vc[i] = krow[i];
+  // optional packed copy of this step's rotated keys and values,
+  // [T, 2, G, D] (needs Dv == D): the dense prefill kernel reads it
+  T* fk = kv_fresh ? kv_fresh + (((int64_t)t * 2 + 0) * G + g) * D : nullptr;
+  T* fv = kv_fresh ? kv_fresh + (((int64_t)t * 2 + 1) * G + g) * D : nullptr;
+  const T* vrow = v != nullptr ? v + (int64_t)t * v_stride + (int64_t)g * Dv : krow;
+  for (int i = threadIdx.x; i < Dv; i += blockDim.x) {
+    vc[i] = vrow[i];
+    if (fv) fv[i] = vrow[i];
   }
   for (int i = threadIdx.x; i < R; i += blockDim.x) {
     float s, c;
@@ -47,8 +50,12 @@ __global__ void rope_pairs_store_kernel(T* __restrict__ q, const T* __restrict__
     const float u = ldf(krow + 2 * i), w = ldf(krow + 2 * i + 1);
     stf(kc + 2 * i, u * c - w * s);
     stf(kc + 2 * i + 1, w * c + u * s);
+    if (fk) { fk[2 * i] = kc[2 * i]; fk[2 * i + 1] = kc[2 * i + 1]; }
   }
-  for (int i = 2 * R + threadIdx.x; i < D; i += blockDim.x) kc[i] = krow[i];
+  for (int i = 2 * R + threadIdx.x; i < D; i += blockDim.x) {
+    kc[i] = krow[i];
+    if (fk) fk[i] = krow[i];
+  }
 }
 
 // grid (T, H), one wave per (query row, head). Keys lo..p, lo = the start of
@@ -63,14 +70,18 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
                                              const int* __restrict__ block_tables,
                                              const int* __restrict__ token_seg,
                                              const int64_t* __restrict__ positions,
-                                             const T* __restrict__ gate, float scale, int mask_size,
+                                             const T* __restrict__ gate, const int* __restrict__ row_map,
+                                             float scale, int mask_size,
                                              int H, int G, int D, int Dv, int BS, int bt_stride,
                                              int q_stride, int gate_stride) {
   extern __shared__ float lds[];       // q [D] | p [64] | key row index [64] (as int)
   float* qs = lds;
   float* ps = lds + D;
   int* rows = (int*)(ps + WAVE);
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  // row_map (optional): the rows this launch serves; the others belong to
+  // the dense prefill kernel
+  const int t = row_map ? row_map[blockIdx.x] : blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
   const int g = h / (H / G);
   const int p = (int)positions[t];
   const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
@@ -126,28 +137,55 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
   }
 }
 
+// out[t, h, :] *= sigmoid(gate[t, h]) — the per-head output gate for rows
+// whose attention came from a kernel without it
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ out, const T* __restrict__ gate, int64_t n, int H, int Dv,
+                                 int gate_stride) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t th = i / Dv;
+    const int64_t t = th / H;
+    const int h = (int)(th - t * H);
+    stf(out + i, ldf(out + i) * sigmoid_exact(ldf(gate + t * gate_stride + h)));
+  }
+}
+
 #define DISPATCH_T(is_f32, ...)                                  \
   if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
 
 extern "C" void seq_launch_rope_pairs_store(void* q, const void* k, const void* v, const int64_t* positions,
                                             const float* inv_freq, void* k_cache, void* v_cache,
-                                            const int64_t* slots, int T_, int H, int G, int D, int Dv, int R,
+                                            const int64_t* slots, void* kv_fresh, int T_, int H, int G, int D,
+                                            int Dv, int R,
                                             int BS, int q_stride, int k_stride, int v_stride, int is_f32,
                                             hipStream_t st) {
   DISPATCH_T(is_f32, hipLaunchKernelGGL(rope_pairs_store_kernel<T>, dim3(T_, H + G), dim3(WAVE), 0, st,
                                         (T*)q, (const T*)k, (const T*)v, positions, inv_freq, (T*)k_cache,
-                                        (T*)v_cache, slots, H, G, D, Dv, R, BS, q_stride, k_stride, v_stride);)
+                                        (T*)v_cache, slots, (T*)kv_fresh, H, G, D, Dv, R, BS, q_stride, k_stride,
+                                        v_stride);)
 }
 
 extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const void* k_cache,
                                                  const void* v_cache, const int* block_tables,
                                                  const int* token_seg, const int64_t* positions,
-                                                 const void* gate, float scale, int mask_size, int T_, int H,
+                                                 const void* gate, const int* row_map, int n_rows,
+                                                 float scale, int mask_size, int T_, int H,
                                                  int G, int D, int Dv, int BS, int bt_stride, int q_stride,
                                                  int gate_stride, int is_f32, hipStream_t st) {
   const size_t lds = (size_t)(D + 2 * WAVE) * sizeof(float);
-  DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(T_, H), dim3(WAVE), lds, st,
+  const int rows = row_map ? n_rows : T_;
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(rows, H), dim3(WAVE), lds, st,
                                         (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
-                                        block_tables, token_seg, positions, (const T*)gate, scale, mask_size,
+                                        block_tables, token_seg, positions, (const T*)gate, row_map, scale,
+                                        mask_size,
                                         H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
+}
+
+extern "C" void seq_launch_head_gate(void* out, const void* gate, int T_, int H, int Dv, int gate_stride,
+                                     int is_f32, hipStream_t st) {
+  const int64_t n = (int64_t)T_ * H * Dv;
+  const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(head_gate_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
+                                        (const T*)gate, n, H, Dv, gate_stride);)
 }

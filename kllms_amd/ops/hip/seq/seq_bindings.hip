@@ -5,6 +5,7 @@
 
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
+#include <hip/hip_bf16.h>
 
 extern "C" {
 void seq_launch_embed_rmsnorm(float*, const int64_t*, const void*, const float*, int, int, float, int, hipStream_t);
@@ -15,20 +16,27 @@ void seq_launch_gated_rmsnorm(void*, const float*, const float*, const void*, in
                               hipStream_t);
 void seq_launch_clamped_glu(void*, const void*, const void*, int64_t, int, int, float, float, int, hipStream_t);
 void seq_launch_rope_pairs_store(void*, const void*, const void*, const int64_t*, const float*, void*, void*,
-                                 const int64_t*, int, int, int, int, int, int, int, int, int, int, int,
+                                 const int64_t*, void*, int, int, int, int, int, int, int, int, int, int, int,
                                  hipStream_t);
 void seq_launch_attn_blocklocal_paged(void*, const void*, const void*, const void*, const int*, const int*,
-                                      const int64_t*, const void*, float, int, int, int, int, int, int, int,
-                                      int, int, int, int, hipStream_t);
+                                      const int64_t*, const void*, const int*, int, float, int, int, int, int,
+                                      int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_head_gate(void*, const void*, int, int, int, int, int, hipStream_t);
 void seq_launch_linear_attn_decay(float*, const void*, const void*, const void*, const float*, float*,
                                   const int*, const int*, const int*, int, int, int, int, int, int, int, int,
                                   hipStream_t);
 void seq_launch_causal_conv_silu(void*, const void*, const float*, void*, const int*, const int*, const int*,
                                  const int*, int, int, int, int, int, int, hipStream_t);
 void seq_launch_gated_delta_rule(float*, const void*, const void*, const void*, const void*, const void*,
-                                 const float*, const float*, float*, const int*, const int*, const int*, int,
-                                 int, int, int, int, int, int, int, int, int, int, hipStream_t);
+                                 const float*, const float*, float*, float*, const int*, const int*, const int*,
+                                 int, int, int, int, int, int, int, int, int, int, int, int, hipStream_t);
 }
+
+// dense varlen causal MFMA prefill kernel (ops/hip/attn_prefill.hip, also part
+// of kllms_amd._C): bf16, head size 128, 8 q-tiles of 32 rows per workgroup
+extern "C" __global__ void attn_prefill_kernel(__hip_bfloat16*, const __hip_bfloat16*, const __hip_bfloat16*,
+                                               const __hip_bfloat16*, const int*, const int*, const int*, float,
+                                               int, int, int, int);
 
 static inline hipStream_t cur_stream() { return at::hip::getCurrentHIPStream().stream(); }
 
@@ -117,7 +125,7 @@ void clamped_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up, double
 // caches: [NB, G, BS, D] / [NB, G, BS, Dv]; v: empty = store the un-rotated key as the value
 void rope_pairs_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor positions,
                       torch::Tensor inv_freq, torch::Tensor k_cache, torch::Tensor v_cache,
-                      torch::Tensor slots) {
+                      torch::Tensor slots, torch::Tensor kv_fresh) {
   CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_SAME(k, q); CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q);
   CHECK_I64C(positions); CHECK_I64C(slots); CHECK_F32C(inv_freq);
   TORCH_CHECK(k.is_cuda() && k_cache.is_cuda() && v_cache.is_cuda() && k_cache.is_contiguous() &&
@@ -135,17 +143,24 @@ void rope_pairs_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::
   } else {
     TORCH_CHECK(Dv == D, "values-from-keys needs equal key and value sizes");
   }
+  const bool fresh = kv_fresh.numel() > 0;
+  if (fresh) {
+    CHECK_SAME(kv_fresh, q);
+    TORCH_CHECK(kv_fresh.is_cuda() && kv_fresh.is_contiguous() && Dv == D &&
+                kv_fresh.numel() == (int64_t)T * 2 * G * D, "kv_fresh must be [T, 2, G, D]");
+  }
   if (T == 0) return;
   seq_launch_rope_pairs_store(q.data_ptr(), k.data_ptr(), has_v ? v.data_ptr() : nullptr,
                               positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(), k_cache.data_ptr(),
-                              v_cache.data_ptr(), slots.data_ptr<int64_t>(), T, H, G, D, Dv, R, BS,
+                              v_cache.data_ptr(), slots.data_ptr<int64_t>(), fresh ? kv_fresh.data_ptr() : nullptr,
+                              T, H, G, D, Dv, R, BS,
                               (int)q.stride(0), (int)k.stride(0), has_v ? (int)v.stride(0) : 0, f32flag(q),
                               cur_stream());
 }
 
 void attn_blocklocal_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
                            torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
-                           torch::Tensor gate, double scale, int64_t mask_size) {
+                           torch::Tensor gate, double scale, int64_t mask_size, torch::Tensor row_map) {
   CHECK_ACT(q); CHECK_ROWS3(q); CHECK_SAME(out, q); CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q);
   CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && k_cache.is_cuda() && v_cache.is_cuda() &&
@@ -159,13 +174,48 @@ void attn_blocklocal_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_c
     CHECK_ROWS2(gate); CHECK_SAME(gate, q);
     TORCH_CHECK(gate.is_cuda() && gate.size(0) == T && gate.size(1) == H);
   }
+  const bool mapped = row_map.numel() > 0;
+  if (mapped) { CHECK_I32C(row_map); TORCH_CHECK(row_map.numel() <= T); }
   if (T == 0) return;
   seq_launch_attn_blocklocal_paged(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                    block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
                                    positions.data_ptr<int64_t>(), has_gate ? gate.data_ptr() : nullptr,
+                                   mapped ? row_map.data_ptr<int>() : nullptr, (int)row_map.numel(),
                                    (float)scale, (int)mask_size, T, H, G, D, Dv, BS,
                                    (int)block_tables.stride(0), (int)q.stride(0),
                                    has_gate ? (int)gate.stride(0) : 0, f32flag(q), cur_stream());
+}
+
+void head_gate(torch::Tensor out, torch::Tensor gate) {
+  CHECK_ACT(out); CHECK_ROWS2(gate); CHECK_SAME(gate, out);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && gate.is_cuda() && gate.size(0) == out.size(0) &&
+              gate.size(1) == out.size(1));
+  if (out.numel() == 0) return;
+  seq_launch_head_gate(out.data_ptr(), gate.data_ptr(), (int)out.size(0), (int)out.size(1), (int)out.size(2),
+                       (int)gate.stride(0), f32flag(out), cur_stream());
+}
+
+// Dense causal attention over packed pieces (each piece attends within
+// itself only): q [T,H,128], k/v [T,G,128] row views with one token stride,
+// bf16. grp_*: q-tile groups built on the host (8 tiles of 32 rows per
+// workgroup, -1 = idle wave). Rows outside every piece are left untouched.
+void attn_varlen_mfma(torch::Tensor out, torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                      torch::Tensor grp_start, torch::Tensor grp_qpos0, torch::Tensor grp_len, double scale) {
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == at::kBFloat16, "bf16 only");
+  CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q); CHECK_SAME(out, q);
+  CHECK_I32C(grp_start); CHECK_I32C(grp_qpos0); CHECK_I32C(grp_len);
+  const int H = q.size(1), D = q.size(2), G = k.size(1);
+  TORCH_CHECK(D == 128 && v.size(2) == 128 && k.size(2) == 128, "head size must be 128");
+  TORCH_CHECK(H % G == 0 && v.size(1) == G && k.stride(0) == v.stride(0), "k/v must share heads and token stride");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.numel() == q.size(0) * (int64_t)H * D);
+  const int ngroups = grp_start.numel();
+  TORCH_CHECK(grp_qpos0.numel() == (int64_t)ngroups * 8 && grp_len.numel() == ngroups);
+  if (ngroups == 0) return;
+  hipLaunchKernelGGL(attn_prefill_kernel, dim3(ngroups, H), dim3(512), 0, cur_stream(),
+                     (__hip_bfloat16*)out.data_ptr(), (const __hip_bfloat16*)q.data_ptr(),
+                     (const __hip_bfloat16*)k.data_ptr(), (const __hip_bfloat16*)v.data_ptr(),
+                     grp_start.data_ptr<int>(), grp_len.data_ptr<int>(), grp_qpos0.data_ptr<int>(), (float)scale,
+                     H, G, (int)q.stride(0), (int)k.stride(0));
 }
 
 static void check_segments(const torch::Tensor& slots, const torch::Tensor& cu, const torch::Tensor& seg_start,
@@ -223,11 +273,14 @@ void gated_delta_rule(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == V);
   TORCH_CHECK(dt_bias.numel() == (int64_t)H * D && a_log.numel() == H && o.numel() == (int64_t)T * H * V);
   if (T == 0 || B == 0) return;
+  // per-(token, head, channel) decays, computed in a parallel pre-pass
+  auto gdec = torch::empty({(int64_t)T, (int64_t)H * D}, torch::dtype(torch::kFloat).device(q.device()));
   seq_launch_gated_delta_rule(o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(), beta.data_ptr(),
                               a.data_ptr(), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),
-                              state.data_ptr<float>(), slots.data_ptr<int>(), cu.data_ptr<int>(),
-                              seg_start.data_ptr<int>(), B, H, G, D, V, (int)q.stride(0), (int)k.stride(0),
-                              (int)v.stride(0), (int)beta.stride(0), (int)a.stride(0), f32flag(q), cur_stream());
+                              gdec.data_ptr<float>(), state.data_ptr<float>(), slots.data_ptr<int>(),
+                              cu.data_ptr<int>(), seg_start.data_ptr<int>(), T, B, H, G, D, V, (int)q.stride(0),
+                              (int)k.stride(0), (int)v.stride(0), (int)beta.stride(0), (int)a.stride(0),
+                              f32flag(q), cur_stream());
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -238,6 +291,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("clamped_glu", &clamped_glu);
   m.def("rope_pairs_store", &rope_pairs_store);
   m.def("attn_blocklocal_paged", &attn_blocklocal_paged);
+  m.def("head_gate", &head_gate);
+  m.def("attn_varlen_mfma", &attn_varlen_mfma);
   m.def("linear_attn_decay", &linear_attn_decay);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("gated_delta_rule", &gated_delta_rule);

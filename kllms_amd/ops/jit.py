@@ -34,7 +34,8 @@ HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rd
 EXTENSIONS = {
     "_C_seq": {
         "dir": os.path.join(HIP_DIR, "seq"),
-        "kernels": ["seq_norm.hip", "seq_attn.hip", "seq_recurrent.hip"],
+        # the dense MFMA prefill kernel is shared with _C (one source, two modules)
+        "kernels": ["seq_norm.hip", "seq_attn.hip", "seq_recurrent.hip", "../attn_prefill.hip"],
         "bindings": ["seq_bindings.hip"],
         "headers": ["seq_common.h"],
     },
@@ -54,7 +55,8 @@ def module_path(name: str) -> str:
 def source_digest(name: str) -> str:
     ext = EXTENSIONS[name]
     h = hashlib.sha256(" ".join(HIP_FLAGS).encode())
-    for f in ext["headers"] + ext["kernels"] + ext["bindings"]:
+    shared = ["../common.h"] if any(f.startswith("../") for f in ext["kernels"]) else []
+    for f in ext["headers"] + shared + ext["kernels"] + ext["bindings"]:
         with open(os.path.join(ext["dir"], f), "rb") as fh:
             h.update(f.encode() + b"\0" + fh.read())
     return h.hexdigest()
@@ -88,7 +90,7 @@ def build(name: str, verbose: bool = False) -> str:
         jobs: List[List[str]] = []
         objs: List[str] = []
         for f in ext["kernels"] + ext["bindings"]:
-            o = os.path.join(obj_dir, f + ".o")
+            o = os.path.join(obj_dir, os.path.basename(f) + ".o")
             cmd = [_hipcc(), "-c", os.path.join(ext["dir"], f), "-o", o] + HIP_FLAGS
             if f in ext["bindings"]:
                 cmd += torch_inc + torch_def
