@@ -22,14 +22,15 @@ void seq_launch_attn_blocklocal_paged(void*, const void*, const void*, const voi
                                       const int64_t*, const void*, const int*, int, float, int, int, int, int,
                                       int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_head_gate(void*, const void*, int, int, int, int, int, hipStream_t);
-void seq_launch_linear_attn_decay(float*, const void*, const void*, const void*, const float*, float*,
+void seq_launch_linear_attn_decay(float*, const void*, const void*, const void*, const float*, float*, float*,
                                   const int*, const int*, const int*, int, int, int, int, int, int, int, int,
-                                  hipStream_t);
+                                  int, hipStream_t);
 void seq_launch_causal_conv_silu(void*, const void*, const float*, void*, const int*, const int*, const int*,
                                  const int*, int, int, int, int, int, int, hipStream_t);
 void seq_launch_gated_delta_rule(float*, const void*, const void*, const void*, const void*, const void*,
-                                 const float*, const float*, float*, float*, const int*, const int*, const int*,
-                                 int, int, int, int, int, int, int, int, int, int, int, int, hipStream_t);
+                                 const float*, const float*, float*, float*, float*, float*, float*, float*,
+                                 const int*, const int*, const int*, int, int, int, int, int, int, int, int, int,
+                                 int, int, int, hipStream_t);
 }
 
 // dense varlen causal MFMA prefill kernel (ops/hip/attn_prefill.hip, also part
@@ -237,10 +238,13 @@ void linear_attn_decay(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch:
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == V);
   TORCH_CHECK(decay.numel() == H && o.numel() == (int64_t)T * H * V);
   if (T == 0 || B == 0) return;
+  // silu(q) | silu(k) | silu(v) per (token, head), fp32, from the parallel pre-pass
+  auto packed = torch::empty({(int64_t)T, (int64_t)H * (2 * D + V)}, torch::dtype(torch::kFloat).device(q.device()));
   seq_launch_linear_attn_decay(o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                               decay.data_ptr<float>(), state.data_ptr<float>(), slots.data_ptr<int>(),
-                               cu.data_ptr<int>(), seg_start.data_ptr<int>(), B, H, D, V, (int)q.stride(0),
-                               (int)k.stride(0), (int)v.stride(0), f32flag(q), cur_stream());
+                               decay.data_ptr<float>(), packed.data_ptr<float>(), state.data_ptr<float>(),
+                               slots.data_ptr<int>(), cu.data_ptr<int>(), seg_start.data_ptr<int>(), T, B, H, D,
+                               V, (int)q.stride(0), (int)k.stride(0), (int)v.stride(0), f32flag(q),
+                               cur_stream());
 }
 
 void causal_conv_silu(torch::Tensor y, torch::Tensor x, torch::Tensor w, torch::Tensor conv_state,
@@ -273,11 +277,17 @@ void gated_delta_rule(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == V);
   TORCH_CHECK(dt_bias.numel() == (int64_t)H * D && a_log.numel() == H && o.numel() == (int64_t)T * H * V);
   if (T == 0 || B == 0) return;
-  // per-(token, head, channel) decays, computed in a parallel pre-pass
-  auto gdec = torch::empty({(int64_t)T, (int64_t)H * D}, torch::dtype(torch::kFloat).device(q.device()));
+  // fp32 operands of the recurrence, from the parallel pre-pass: unit q and k,
+  // per-channel decays, values, write strengths
+  auto f32 = torch::dtype(torch::kFloat).device(q.device());
+  auto qn = torch::empty({(int64_t)T, (int64_t)G * D}, f32), kn = torch::empty({(int64_t)T, (int64_t)G * D}, f32);
+  auto gd = torch::empty({(int64_t)T, (int64_t)H * D}, f32), vf = torch::empty({(int64_t)T, (int64_t)H * V}, f32);
+  auto bt = torch::empty({(int64_t)T, (int64_t)H}, f32);
   seq_launch_gated_delta_rule(o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(), beta.data_ptr(),
                               a.data_ptr(), dt_bias.data_ptr<float>(), a_log.data_ptr<float>(),
-                              gdec.data_ptr<float>(), state.data_ptr<float>(), slots.data_ptr<int>(),
+                              qn.data_ptr<float>(), kn.data_ptr<float>(), gd.data_ptr<float>(),
+                              vf.data_ptr<float>(), bt.data_ptr<float>(), state.data_ptr<float>(),
+                              slots.data_ptr<int>(),
                               cu.data_ptr<int>(), seg_start.data_ptr<int>(), T, B, H, G, D, V, (int)q.stride(0),
                               (int)k.stride(0), (int)v.stride(0), (int)beta.stride(0), (int)a.stride(0),
                               f32flag(q), cur_stream());

@@ -4,70 +4,120 @@
 // starts a sequence (seg_start == 0) takes its state as zero whatever the
 // slot holds, so a reused slot needs no clearing.
 //
-// Layout of the recurrences: one wave per (segment, head, 64 state columns);
-// lane j owns one column of the state (D floats in registers) — the per-token
-// update and read-out are then lane-local, and the slot traffic is coalesced
-// over j. Splitting the columns over waves keeps a lone long prompt from
-// running on H workgroups only.
+// Layout of the recurrences: one wave per (segment, head, 32 state columns).
+// The two half-waves split the state's rows: lane (half, j) keeps rows
+// half*D/2 .. of column j in registers, so the per-token update is lane-local
+// and the read-out needs one exchange between the halves; slot traffic is
+// coalesced over j. Splitting columns and rows over many small waves keeps a
+// few long prompts from running on a handful of SIMDs.
 
 #include "seq_common.h"
 
 // ---- decayed linear attention ------------------------------------------------
 // S <- decay_h S + silu(k) silu(v)^T ; o = S^T silu(q)
-template <typename T, int DMAX>
+//
+// Two kernels. A parallel pre-pass applies silu and packs q|k|v per (token,
+// head) in fp32; the recurrence then only loads and multiplies. One wave of
+// the recurrence serves (segment, head, 64/NS state columns): its NS lane
+// groups split the state's rows (DMAX/NS each, in registers), so the update is
+// lane-local and the read-out is reduced over the groups with NS-1 exchanges.
+// A single wave issues slowly on this hardware; NS is chosen at launch so that
+// there are several waves per SIMD even for a few long prompts.
+template <typename T>
+__global__ void linear_prep_kernel(float* __restrict__ pk, const T* __restrict__ q,
+                                   const T* __restrict__ k, const T* __restrict__ v, int64_t n, int H,
+                                   int D, int V, int q_stride, int k_stride, int v_stride) {
+  const int W = 2 * D + V;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t th = i / W;
+    const int c = (int)(i - th * W);
+    const int64_t t = th / H;
+    const int h = (int)(th - t * H);
+    float x;
+    if (c < D) x = ldf(q + t * q_stride + (int64_t)h * D + c);
+    else if (c < 2 * D) x = ldf(k + t * k_stride + (int64_t)h * D + (c - D));
+    else x = ldf(v + t * v_stride + (int64_t)h * V + (c - 2 * D));
+    pk[i] = silu_exact(x);
+  }
+}
+
+template <int DMAX, int NS>
 __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
-    float* __restrict__ o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-    const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ slots,
-    const int* __restrict__ cu, const int* __restrict__ seg_start, int H, int D, int V,
-    int q_stride, int k_stride, int v_stride) {
-  constexpr int PER = (2 * DMAX + WAVE - 1) / WAVE;     // q|k elements staged per lane
-  __shared__ float qk[2][2 * DMAX];
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, j = blockIdx.z * WAVE + lane;
+    float* __restrict__ o, const float* __restrict__ pk, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ cu,
+    const int* __restrict__ seg_start, int H, int D, int V) {
+  constexpr int TB = 4;                                   // tokens per pipeline stage
+  constexpr int DR = DMAX / NS, COLS = WAVE / NS;         // state rows / columns per lane group
+  constexpr int PER = (2 * DMAX + WAVE - 1) / WAVE;       // q|k elements staged per lane
+  __shared__ float qk[2][TB][2 * DMAX];
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int grp = lane / COLS, j = blockIdx.z * COLS + (lane % COLS), d0 = grp * DR;
   const bool live = j < V;
   const int t0 = cu[b], t1 = cu[b + 1];
+  const int W = 2 * D + V;
   float* sp = state + (((int64_t)slots[b] * H + h) * D) * V + j;
-  float S[DMAX];
+  float S[DR];
   const bool fresh = seg_start[b] == 0;
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = (!fresh && live && d < D) ? sp[(int64_t)d * V] : 0.f;
+  for (int d = 0; d < DR; ++d) S[d] = (!fresh && live && d0 + d < D) ? sp[(int64_t)(d0 + d) * V] : 0.f;
   const float dec = decay[h];
-  // software pipeline: token t+1's q, k, v are in flight while token t is computed
-  float pre[PER], vpre = 0.f;
-  auto fetch = [&](int t) {
+  // rows D..DMAX-1 of the staging buffers stay zero, so the unrolled loops
+  // below run over DMAX without a bound check (a branch per row would keep
+  // the LDS reads from being batched)
+  for (int i = lane; i < 2 * TB * 2 * DMAX; i += WAVE) (&qk[0][0][0])[i] = 0.f;
+  __syncthreads();
+  // software pipeline over groups of TB tokens: the next group's operands are
+  // in flight while this group's tokens are computed one after the other
+  float pre[TB][PER], vpre[TB];
+  auto fetch = [&](int tg) {
 #pragma unroll
-    for (int r = 0; r < PER; ++r) {
-      const int i = lane + r * WAVE;
-      const bool isq = i < D;
-      const int d = isq ? i : i - D;
-      pre[r] = i < 2 * D ? ldf((isq ? q + (int64_t)t * q_stride : k + (int64_t)t * k_stride) + (int64_t)h * D + d)
-                         : 0.f;
+    for (int u = 0; u < TB; ++u) {
+      const int t = tg + u;
+      const bool on = t < t1;
+      const float* row = pk + ((int64_t)t * H + h) * W;
+#pragma unroll
+      for (int r = 0; r < PER; ++r) {
+        const int i = lane + r * WAVE;
+        pre[u][r] = (on && i < 2 * D) ? row[i] : 0.f;
+      }
+      vpre[u] = (on && live) ? row[2 * D + j] : 0.f;
     }
-    vpre = live ? ldf(v + (int64_t)t * v_stride + (int64_t)h * V + j) : 0.f;
   };
   if (t0 < t1) fetch(t0);
-  for (int t = t0; t < t1; ++t) {
-    float* buf = qk[(t - t0) & 1];
+  int flip = 0;
+  for (int tg = t0; tg < t1; tg += TB, flip ^= 1) {
+    float vj[TB];
 #pragma unroll
-    for (int r = 0; r < PER; ++r) {
-      const int i = lane + r * WAVE;
-      if (i < 2 * D) buf[i < D ? i : DMAX + (i - D)] = silu_exact(pre[r]);
+    for (int u = 0; u < TB; ++u) {
+#pragma unroll
+      for (int r = 0; r < PER; ++r) {
+        const int i = lane + r * WAVE;
+        if (i < 2 * D) qk[flip][u][i < D ? i : DMAX + (i - D)] = pre[u][r];
+      }
+      vj[u] = vpre[u];
     }
-    const float vj = silu_exact(vpre);
-    __syncthreads();    // double-buffered: one barrier per token
-    if (t + 1 < t1) fetch(t + 1);
-    float acc = 0.f;
+    __syncthreads();    // double-buffered: one barrier per group
+    if (tg + TB < t1) fetch(tg + TB);
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
-        S[d] = dec * S[d] + buf[DMAX + d] * vj;
-        acc += S[d] * buf[d];
+    for (int u = 0; u < TB; ++u) {
+      if (tg + u < t1) {
+        const float* buf = qk[flip][u];
+        float acc = 0.f;
+#pragma unroll
+        for (int d = 0; d < DR; ++d) {
+          S[d] = dec * S[d] + buf[DMAX + d0 + d] * vj[u];
+          acc += S[d] * buf[d0 + d];
+        }
+#pragma unroll
+        for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
+        if (live && grp == 0) o[((int64_t)(tg + u) * H + h) * V + j] = acc;
       }
     }
-    if (live) o[((int64_t)t * H + h) * V + j] = acc;
   }
   if (live) {
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) if (d < D) sp[(int64_t)d * V] = S[d];
+    for (int d = 0; d < DR; ++d) if (d0 + d < D) sp[(int64_t)(d0 + d) * V] = S[d];
   }
 }
 
@@ -128,95 +178,137 @@ __global__ void conv_state_update_kernel(const T* __restrict__ x, T* __restrict_
 // per token: g_d = exp(-exp(A_h) softplus(a_d + dt_d));  S <- g (.) S (rows)
 //            u = beta (v - S^T k^) ; S <- S + k^ u^T ; o = S^T q^
 // k^ = k / sqrt(|k|^2 + 1e-6), q^ likewise times D^-1/2; beta = sigmoid(.)
-// decay pre-pass, parallel over all (token, head, channel):
-//   g = exp(-exp(A_h) softplus(a + dt))
+// Pre-pass, parallel over tokens — one wave per (token, q/k head) and one per
+// (token, value head):
+//   qn = q / sqrt(|q|^2 + 1e-6) * D^-1/2,  kn = k / sqrt(|k|^2 + 1e-6)     [T, G, D] fp32
+//   g  = exp(-exp(A_h) softplus(a + dt))                                    [T, H, D] fp32
+//   vf = v, beta = sigmoid(b)                                              [T, H, V], [T, H] fp32
 template <typename T>
-__global__ void delta_decay_kernel(float* __restrict__ g, const T* __restrict__ a,
-                                   const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                                   int64_t n, int HD, int D, int a_stride) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t t = i / HD;
-    const int c = (int)(i - t * HD);
-    const float pre = ldf(a + t * a_stride + c) + dt_bias[c];
-    g[i] = expf(-expf(a_log[c / D]) * softplus_exact(pre));
+__global__ void delta_prep_kernel(float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ gd,
+                                  float* __restrict__ vf, float* __restrict__ bt, const T* __restrict__ q,
+                                  const T* __restrict__ k, const T* __restrict__ v,
+                                  const T* __restrict__ beta_logit, const T* __restrict__ a,
+                                  const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                                  int H, int G, int D, int V, int q_stride, int k_stride, int v_stride,
+                                  int beta_stride, int a_stride) {
+  const int64_t t = blockIdx.x;
+  const int y = blockIdx.y, lane = threadIdx.x;
+  if (y < G) {
+    const T* qr = q + t * q_stride + (int64_t)y * D;
+    const T* kr = k + t * k_stride + (int64_t)y * D;
+    float sq = 0.f, sk = 0.f;
+    for (int d = lane; d < D; d += WAVE) {
+      const float x = ldf(qr + d), z = ldf(kr + d);
+      sq += x * x; sk += z * z;
+    }
+    sq = wave_sum(sq); sk = wave_sum(sk);
+    const float rq = 1.0f / (sqrtf(sq + 1e-6f) * sqrtf((float)D)), rk = 1.0f / sqrtf(sk + 1e-6f);
+    for (int d = lane; d < D; d += WAVE) {
+      qn[(t * G + y) * D + d] = ldf(qr + d) * rq;
+      kn[(t * G + y) * D + d] = ldf(kr + d) * rk;
+    }
+  } else {
+    const int h = y - G;
+    const float rate = expf(a_log[h]);
+    for (int d = lane; d < D; d += WAVE) {
+      const float pre = ldf(a + t * a_stride + (int64_t)h * D + d) + dt_bias[(int64_t)h * D + d];
+      gd[(t * H + h) * D + d] = expf(-rate * softplus_exact(pre));
+    }
+    for (int i = lane; i < V; i += WAVE) vf[(t * H + h) * V + i] = ldf(v + t * v_stride + (int64_t)h * V + i);
+    if (lane == 0) bt[t * H + h] = sigmoid_exact(ldf(beta_logit + t * beta_stride + h));
   }
 }
 
-template <typename T, int DMAX>
+// The recurrence proper, on the pre-pass's fp32 operands; wave layout and
+// pipeline as in linear_attn_decay_kernel.
+template <int DMAX, int NS>
 __global__ void __launch_bounds__(WAVE) gated_delta_rule_kernel(
-    float* __restrict__ o, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-    const T* __restrict__ beta_logit, const float* __restrict__ gdec, float* __restrict__ state,
-    const int* __restrict__ slots, const int* __restrict__ cu, const int* __restrict__ seg_start,
-    int H, int G, int D, int V, int q_stride, int k_stride, int v_stride, int beta_stride) {
-  constexpr int PER = (3 * DMAX + WAVE - 1) / WAVE;     // q|k|g elements staged per lane
-  __shared__ float buf_[2][3 * DMAX];
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, j = blockIdx.z * WAVE + lane;
+    float* __restrict__ o, const float* __restrict__ qn, const float* __restrict__ kn,
+    const float* __restrict__ gd, const float* __restrict__ vf, const float* __restrict__ bt,
+    float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ cu,
+    const int* __restrict__ seg_start, int H, int G, int D, int V) {
+  constexpr int TB = 4;
+  constexpr int DR = DMAX / NS, COLS = WAVE / NS;
+  constexpr int PER = (3 * DMAX + WAVE - 1) / WAVE;       // q|k|g elements staged per lane
+  __shared__ float buf_[2][TB][3 * DMAX];
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int grp = lane / COLS, j = blockIdx.z * COLS + (lane % COLS), d0 = grp * DR;
   const int g = h / (H / G);
   const bool live = j < V;
   const int t0 = cu[b], t1 = cu[b + 1];
   float* sp = state + (((int64_t)slots[b] * H + h) * D) * V + j;
-  float S[DMAX];
+  float S[DR];
   const bool fresh = seg_start[b] == 0;
 #pragma unroll
-  for (int d = 0; d < DMAX; ++d) S[d] = (!fresh && live && d < D) ? sp[(int64_t)d * V] : 0.f;
-  const float qscale = 1.0f / sqrtf((float)D);
-  // software pipeline: token t+1's operands are in flight while token t is computed
-  float pre[PER], vpre = 0.f, bpre = 0.f;
-  auto fetch = [&](int t) {
+  for (int d = 0; d < DR; ++d) S[d] = (!fresh && live && d0 + d < D) ? sp[(int64_t)(d0 + d) * V] : 0.f;
+  for (int i = lane; i < 2 * TB * 3 * DMAX; i += WAVE) (&buf_[0][0][0])[i] = 0.f;   // pad rows stay zero
+  __syncthreads();
+  float pre[TB][PER], vpre[TB], bpre[TB];
+  // where each staged element comes from and goes to, fixed per lane: element
+  // i = lane + r*64 of q|k|g (no index division inside the token loop)
+  const float* src[PER];
+  int src_step[PER], dst[PER];
 #pragma unroll
-    for (int r = 0; r < PER; ++r) {
-      const int i = lane + r * WAVE;
-      const int which = i / D, d = i - which * D;
-      float val = 0.f;
-      if (which == 0) val = ldf(q + (int64_t)t * q_stride + (int64_t)g * D + d);
-      else if (which == 1) val = ldf(k + (int64_t)t * k_stride + (int64_t)g * D + d);
-      else if (which == 2) val = gdec[((int64_t)t * H + h) * D + d];
-      pre[r] = val;
+  for (int r = 0; r < PER; ++r) {
+    const int i = lane + r * WAVE;
+    const int which = i / D, d = i - which * D;
+    dst[r] = which < 3 ? which * DMAX + d : -1;
+    src[r] = which == 0 ? qn + (int64_t)g * D + d : which == 1 ? kn + (int64_t)g * D + d : gd + (int64_t)h * D + d;
+    src_step[r] = which == 2 ? H * D : G * D;
+  }
+  auto fetch = [&](int tg) {
+#pragma unroll
+    for (int u = 0; u < TB; ++u) {
+      const int t = tg + u;
+      const bool on = t < t1;
+#pragma unroll
+      for (int r = 0; r < PER; ++r) pre[u][r] = (on && dst[r] >= 0) ? src[r][(int64_t)t * src_step[r]] : 0.f;
+      vpre[u] = (on && live) ? vf[((int64_t)t * H + h) * V + j] : 0.f;
+      bpre[u] = on ? bt[(int64_t)t * H + h] : 0.f;
     }
-    vpre = live ? ldf(v + (int64_t)t * v_stride + (int64_t)h * V + j) : 0.f;
-    bpre = ldf(beta_logit + (int64_t)t * beta_stride + h);
   };
   if (t0 < t1) fetch(t0);
-  for (int t = t0; t < t1; ++t) {
-    float* buf = buf_[(t - t0) & 1];
+  int flip = 0;
+  for (int tg = t0; tg < t1; tg += TB, flip ^= 1) {
+    float vj[TB], beta[TB];
 #pragma unroll
-    for (int r = 0; r < PER; ++r) {
-      const int i = lane + r * WAVE;
-      const int which = i / D, d = i - which * D;
-      if (which < 3) buf[which * DMAX + d] = pre[r];
+    for (int u = 0; u < TB; ++u) {
+#pragma unroll
+      for (int r = 0; r < PER; ++r)
+        if (dst[r] >= 0) buf_[flip][u][dst[r]] = pre[u][r];
+      vj[u] = vpre[u];
+      beta[u] = bpre[u];
     }
-    const float vj = vpre;
-    const float beta = sigmoid_exact(bpre);
     __syncthreads();
-    if (t + 1 < t1) fetch(t + 1);
-    float pred = 0.f, ksq = 0.f, qsq = 0.f;
+    if (tg + TB < t1) fetch(tg + TB);
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
-        const float kd = buf[DMAX + d], qd = buf[d];
-        S[d] *= buf[2 * DMAX + d];
-        pred += S[d] * kd;
-        ksq += kd * kd;
-        qsq += qd * qd;
+    for (int u = 0; u < TB; ++u) {
+      if (tg + u < t1) {
+        const float* buf = buf_[flip][u];
+        float pred = 0.f;
+#pragma unroll
+        for (int d = 0; d < DR; ++d) {
+          S[d] *= buf[2 * DMAX + d0 + d];
+          pred += S[d] * buf[DMAX + d0 + d];
+        }
+#pragma unroll
+        for (int off = COLS; off < WAVE; off <<= 1) pred += __shfl_xor(pred, off);
+        const float uu = beta[u] * (vj[u] - pred);
+        float acc = 0.f;
+#pragma unroll
+        for (int d = 0; d < DR; ++d) {
+          S[d] += buf[DMAX + d0 + d] * uu;
+          acc += S[d] * buf[d0 + d];
+        }
+#pragma unroll
+        for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
+        if (live && grp == 0) o[((int64_t)(tg + u) * H + h) * V + j] = acc;
       }
     }
-    const float rk = 1.0f / sqrtf(ksq + 1e-6f);
-    const float rq = qscale / sqrtf(qsq + 1e-6f);
-    const float u = beta * (vj - pred * rk) * rk;     // u times the key's normaliser
-    float acc = 0.f;
-#pragma unroll
-    for (int d = 0; d < DMAX; ++d) {
-      if (d < D) {
-        S[d] += buf[DMAX + d] * u;
-        acc += S[d] * buf[d];
-      }
-    }
-    if (live) o[((int64_t)t * H + h) * V + j] = acc * rq;
   }
   if (live) {
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) if (d < D) sp[(int64_t)d * V] = S[d];
+    for (int d = 0; d < DR; ++d) if (d0 + d < D) sp[(int64_t)(d0 + d) * V] = S[d];
   }
 }
 
@@ -229,17 +321,34 @@ __global__ void __launch_bounds__(WAVE) gated_delta_rule_kernel(
   else if (D <= 128) { constexpr int DMAX = 128; __VA_ARGS__ }      \
   else { constexpr int DMAX = 256; __VA_ARGS__ }
 
-static inline int col_blocks(int V) { return (V + WAVE - 1) / WAVE; }
+// rows of the state are split over NS lane groups; more groups = more, smaller
+// waves. Take the coarsest split that still gives ~4 waves per SIMD.
+static inline int pick_split(int B, int H, int V) {
+  const int64_t want = 4096;
+  for (int ns = 2; ns <= 8; ns *= 2)
+    if ((int64_t)B * H * ((V + 64 / ns - 1) / (64 / ns)) >= want) return ns;
+  return 8;
+}
+
+#define DISPATCH_NS(ns, ...)                                        \
+  if (ns == 2) { constexpr int NS = 2; __VA_ARGS__ }                \
+  else if (ns == 4) { constexpr int NS = 4; __VA_ARGS__ }           \
+  else { constexpr int NS = 8; __VA_ARGS__ }
 
 extern "C" void seq_launch_linear_attn_decay(float* o, const void* q, const void* k, const void* v,
-                                             const float* decay, float* state, const int* slots,
-                                             const int* cu, const int* seg_start, int B, int H, int D, int V,
-                                             int q_stride, int k_stride, int v_stride, int is_f32,
-                                             hipStream_t st) {
-  DISPATCH_T(is_f32, DISPATCH_D(D, hipLaunchKernelGGL((linear_attn_decay_kernel<T, DMAX>), dim3(B, H, col_blocks(V)),
-                                                      dim3(WAVE), 0, st, o, (const T*)q,
-                                                      (const T*)k, (const T*)v, decay, state, slots, cu,
-                                                      seg_start, H, D, V, q_stride, k_stride, v_stride);))
+                                             const float* decay, float* packed, float* state,
+                                             const int* slots, const int* cu, const int* seg_start, int T_,
+                                             int B, int H, int D, int V, int q_stride, int k_stride,
+                                             int v_stride, int is_f32, hipStream_t st) {
+  const int64_t n = (int64_t)T_ * H * (2 * D + V);
+  const int grid = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(linear_prep_kernel<T>, dim3(grid), dim3(256), 0, st, packed,
+                                        (const T*)q, (const T*)k, (const T*)v, n, H, D, V, q_stride, k_stride,
+                                        v_stride);)
+  const int ns = pick_split(B, H, V);
+  DISPATCH_NS(ns, DISPATCH_D(D, hipLaunchKernelGGL((linear_attn_decay_kernel<DMAX, NS>),
+                                                   dim3(B, H, (V + WAVE / NS - 1) / (WAVE / NS)), dim3(WAVE), 0,
+                                                   st, o, packed, decay, state, slots, cu, seg_start, H, D, V);))
 }
 
 extern "C" void seq_launch_causal_conv_silu(void* y, const void* x, const float* w, void* conv_state,
@@ -258,17 +367,18 @@ extern "C" void seq_launch_causal_conv_silu(void* y, const void* x, const float*
 
 extern "C" void seq_launch_gated_delta_rule(float* o, const void* q, const void* k, const void* v,
                                             const void* beta_logit, const void* a, const float* dt_bias,
-                                            const float* a_log, float* gdec, float* state, const int* slots,
-                                            const int* cu, const int* seg_start, int T_, int B, int H, int G,
-                                            int D, int V, int q_stride, int k_stride, int v_stride,
-                                            int beta_stride, int a_stride, int is_f32, hipStream_t st) {
-  const int64_t n = (int64_t)T_ * H * D;
-  const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
-  DISPATCH_T(is_f32,
-             hipLaunchKernelGGL(delta_decay_kernel<T>, dim3(grid), dim3(256), 0, st, gdec, (const T*)a, dt_bias,
-                                a_log, n, H * D, D, a_stride);
-             DISPATCH_D(D, hipLaunchKernelGGL((gated_delta_rule_kernel<T, DMAX>), dim3(B, H, col_blocks(V)),
-                                              dim3(WAVE), 0, st, o, (const T*)q, (const T*)k, (const T*)v,
-                                              (const T*)beta_logit, gdec, state, slots, cu, seg_start, H, G, D,
-                                              V, q_stride, k_stride, v_stride, beta_stride);))
+                                            const float* a_log, float* qn, float* kn, float* gd, float* vf,
+                                            float* bt, float* state, const int* slots, const int* cu,
+                                            const int* seg_start, int T_, int B, int H, int G, int D, int V,
+                                            int q_stride, int k_stride, int v_stride, int beta_stride,
+                                            int a_stride, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(delta_prep_kernel<T>, dim3(T_, G + H), dim3(WAVE), 0, st, qn, kn, gd,
+                                        vf, bt, (const T*)q, (const T*)k, (const T*)v, (const T*)beta_logit,
+                                        (const T*)a, dt_bias, a_log, H, G, D, V, q_stride, k_stride, v_stride,
+                                        beta_stride, a_stride);)
+  const int ns = pick_split(B, H, V);
+  DISPATCH_NS(ns, DISPATCH_D(D, hipLaunchKernelGGL((gated_delta_rule_kernel<DMAX, NS>),
+                                                   dim3(B, H, (V + WAVE / NS - 1) / (WAVE / NS)), dim3(WAVE), 0,
+                                                   st, o, qn, kn, gd, vf, bt, state, slots, cu, seg_start, H, G,
+                                                   D, V);))
 }
