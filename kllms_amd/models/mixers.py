@@ -265,7 +265,9 @@ class ChannelDeltaMixer(nn.Module):
         self.gd, self.hv = spec.kv_heads * spec.dim, spec.heads * spec.vdim
         self.inp = FusedInput(hidden, [("q", self.gd), ("k", self.gd), ("v", self.hv),
                                        ("a1", spec.decay_rank), ("g1", spec.gate_rank), ("b", spec.heads)], dtype)
-        self.conv = _param(2 * self.gd + self.hv, spec.conv, dtype=torch.float32)
+        # taps-major [K, C] over the q|k|v channels (the checkpoint's [C, K] transposed:
+        # the kernels read 8 channels of one tap at a time)
+        self.conv = _param(spec.conv, 2 * self.gd + self.hv, dtype=torch.float32)
         self.a2 = _param(spec.heads * spec.dim, spec.decay_rank, dtype=dtype)
         self.g2 = _param(self.hv, spec.gate_rank, dtype=dtype)
         self.dt_bias = _param(spec.heads * spec.dim, dtype=torch.float32)
@@ -298,9 +300,9 @@ class ChannelDeltaMixer(nn.Module):
     def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
         m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
         gd = self.gd
-        m[pre + "q.conv"] = self.conv[:gd]
-        m[pre + "k.conv"] = self.conv[gd:2 * gd]
-        m[pre + "v.conv"] = self.conv[2 * gd:]
+        m[pre + "q.conv"] = self.conv.t()[:gd]
+        m[pre + "k.conv"] = self.conv.t()[gd:2 * gd]
+        m[pre + "v.conv"] = self.conv.t()[2 * gd:]
         for n in ("a2", "g2", "dt_bias", "A_log", "norm"):
             m[pre + n] = getattr(self, n)
         m[pre + "o"] = self.o_proj

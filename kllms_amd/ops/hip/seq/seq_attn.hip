@@ -151,6 +151,23 @@ __global__ void head_gate_kernel(T* __restrict__ out, const T* __restrict__ gate
   }
 }
 
+template <typename T>
+__global__ void head_gate_v8_kernel(T* __restrict__ out, const T* __restrict__ gate, int64_t n8, int H, int Dv8,
+                                    int gate_stride) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t th = i / Dv8;
+    const int64_t t = th / H;
+    const int h = (int)(th - t * H);
+    const float s = sigmoid_exact(ldf(gate + t * gate_stride + h));
+    float v[8];
+    ld8(out + i * 8, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= s;
+    st8(out + i * 8, v);
+  }
+}
+
 #define DISPATCH_T(is_f32, ...)                                  \
   if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
 
@@ -185,6 +202,12 @@ extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const
 extern "C" void seq_launch_head_gate(void* out, const void* gate, int T_, int H, int Dv, int gate_stride,
                                      int is_f32, hipStream_t st) {
   const int64_t n = (int64_t)T_ * H * Dv;
+  if (Dv % 8 == 0 && aligned16(out)) {
+    const int g8 = (int)((n / 8 + 255) / 256 < 16384 ? (n / 8 + 255) / 256 : 16384);
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(head_gate_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)out,
+                                          (const T*)gate, n / 8, H, Dv / 8, gate_stride);)
+    return;
+  }
   const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(head_gate_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
                                         (const T*)gate, n, H, Dv, gate_stride);)

@@ -251,8 +251,10 @@ void causal_conv_silu(torch::Tensor y, torch::Tensor x, torch::Tensor w, torch::
                       torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start, torch::Tensor token_seg) {
   CHECK_ACT(x); CHECK_ROWS2(x); CHECK_SAME(y, x); CHECK_SAME(conv_state, x); CHECK_F32C(w); CHECK_I32C(token_seg);
   check_segments(slots, cu, seg_start, conv_state);
-  const int T = x.size(0), C = x.size(1), K = w.size(1), B = slots.numel();
-  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == (int64_t)T * C && w.dim() == 2 && w.size(0) == C);
+  // w: taps-major [K, C], last row = the current token's tap
+  TORCH_CHECK(w.dim() == 2);
+  const int T = x.size(0), C = x.size(1), K = w.size(0), B = slots.numel();
+  TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == (int64_t)T * C && w.size(1) == C);
   TORCH_CHECK(K >= 2 && K <= 16, "2..16 convolution taps supported");
   TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(1) == K - 1 && conv_state.size(2) == C);
   TORCH_CHECK(token_seg.numel() == T);

@@ -44,7 +44,7 @@ __global__ void sandwich_residual_kernel(float* __restrict__ x, const T* __restr
                                          const float* __restrict__ wb, const float* __restrict__ w_post,
                                          const float* __restrict__ w_next, T* __restrict__ out,
                                          int W, float eps) {
-  extern __shared__ float ybuf[];
+  extern __shared__ __align__(16) float ybuf[];
   __shared__ float scratch[16];
   const int64_t base = (int64_t)blockIdx.x * W;
   const float invW = 1.0f / (float)W;
@@ -81,6 +81,67 @@ __global__ void sandwich_residual_kernel(float* __restrict__ x, const T* __restr
   for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + base + i, ybuf[i] * rx * w_next[i]);
 }
 
+// The same epilogue with 8-wide accesses (W % 8 == 0, 16-byte aligned rows).
+template <typename T, bool DUAL>
+__global__ void sandwich_residual_v8_kernel(float* __restrict__ x, const T* __restrict__ a,
+                                            const T* __restrict__ b, const float* __restrict__ wa,
+                                            const float* __restrict__ wb, const float* __restrict__ w_post,
+                                            const float* __restrict__ w_next, T* __restrict__ out,
+                                            int W, float eps) {
+  extern __shared__ __align__(16) float ybuf[];
+  __shared__ float scratch[16];
+  const int64_t base = (int64_t)blockIdx.x * W;
+  const float invW = 1.0f / (float)W;
+  float ssy = 0.f;
+  float va[8], vb[8], w1[8], w2[8], y[8];
+  if (DUAL) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+      ld8(a + base + i, va); ld8(b + base + i, vb);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { sa += va[e] * va[e]; sb += vb[e] * vb[e]; }
+    }
+    sa = block_sum(sa, scratch);
+    sb = block_sum(sb, scratch);
+    const float ra = 1.0f / sqrtf(sa * invW + eps), rb = 1.0f / sqrtf(sb * invW + eps);
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+      ld8(a + base + i, va); ld8(b + base + i, vb); ld8(wa + i, w1); ld8(wb + i, w2);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[e] = 0.5f * (va[e] * ra * w1[e] + vb[e] * rb * w2[e]);
+        ssy += y[e] * y[e];
+      }
+      st8(ybuf + i, y);
+    }
+  } else {
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+      ld8(a + base + i, y);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ssy += y[e] * y[e];
+      st8(ybuf + i, y);
+    }
+  }
+  ssy = block_sum(ssy, scratch);
+  const float ry = 1.0f / sqrtf(ssy * invW + eps);
+  float ssx = 0.f;
+  for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {   // each thread re-reads its own ybuf entries
+    ld8(ybuf + i, y); ld8(x + base + i, va); ld8(w_post + i, w1);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { va[e] += y[e] * ry * w1[e]; ssx += va[e] * va[e]; }
+    st8(x + base + i, va);
+    st8(ybuf + i, va);
+  }
+  if (w_next == nullptr) return;
+  ssx = block_sum(ssx, scratch);
+  const float rx = 1.0f / sqrtf(ssx * invW + eps);
+  for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+    ld8(ybuf + i, va); ld8(w_next + i, w1);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = va[e] * rx * w1[e];
+    st8(out + base + i, y);
+  }
+}
+
 // out[t, g*S + i] = o[t,g,i] / rms(o[t,g,:]) * w[i] * sigmoid(gate[t, g*S + i])
 template <typename T>
 __global__ void gated_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ o,
@@ -99,6 +160,71 @@ __global__ void gated_rmsnorm_kernel(T* __restrict__ out, const float* __restric
     stf(orow + i, row[i] * r * w[i] * sigmoid_exact(ldf(grow + i)));
 }
 
+// 8-wide, single pass: each thread keeps its (up to two) chunks of the row in
+// registers between the sum of squares and the scaling. One workgroup per row.
+template <typename T>
+__global__ void gated_rmsnorm_v8_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                        const float* __restrict__ w, const T* __restrict__ gate,
+                                        int S, int gate_stride, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, g = blockIdx.y, G = gridDim.y;
+  const float* row = o + ((int64_t)t * G + g) * S;
+  float v[2][8], ww[8], gg[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int i = (threadIdx.x + c * blockDim.x) * 8;
+    if (i < S) {
+      ld8(row + i, v[c]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)S + eps);
+  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)g * S;
+  T* orow = out + ((int64_t)t * G + g) * S;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int i = (threadIdx.x + c * blockDim.x) * 8;
+    if (i < S) {
+      ld8(w + i, ww); ld8(grow + i, gg);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[c][e] = v[c][e] * r * ww[e] * sigmoid_exact(gg[e]);
+      st8(orow + i, v[c]);
+    }
+  }
+}
+
+// Short rows (S = 8 * LPG, LPG a power of two <= 64): LPG lanes per row, 64/LPG
+// rows per wave, reduction inside the lane group.
+template <typename T>
+__global__ void gated_rmsnorm_rows_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                          const float* __restrict__ w, const T* __restrict__ gate,
+                                          int64_t rows, int G, int S, int LPG, int gate_stride, float eps) {
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t row = tid / LPG;
+  const int i = (int)(tid - row * LPG) * 8;
+  const bool on = row < rows;
+  float v[8], ww[8], gg[8];
+  float ss = 0.f;
+  if (on) {
+    ld8(o + row * S + i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+  }
+  for (int off = 1; off < LPG; off <<= 1) ss += __shfl_xor(ss, off);
+  if (!on) return;
+  const float r = 1.0f / sqrtf(ss / (float)S + eps);
+  const int64_t t = row / G;
+  const int g = (int)(row - t * G);
+  ld8(w + i, ww);
+  ld8(gate + t * gate_stride + (int64_t)g * S + i, gg);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = v[e] * r * ww[e] * sigmoid_exact(gg[e]);
+  st8(out + row * S + i, v);
+}
+
 // y = min(g, lim) * sigmoid(alpha * min(g, lim)) * (clamp(u, -lim, lim) + 1)
 template <typename T>
 __global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ gate,
@@ -110,6 +236,25 @@ __global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ ga
     float g = fminf(ldf(gate + r * stride + c), limit);
     float u = fminf(fmaxf(ldf(up + r * stride + c), -limit), limit);
     stf(out + i, g * sigmoid_exact(alpha * g) * (u + 1.0f));
+  }
+}
+
+template <typename T>
+__global__ void clamped_glu_v8_kernel(T* __restrict__ out, const T* __restrict__ gate,
+                                      const T* __restrict__ up, int64_t n8, int cols8, int stride,
+                                      float limit, float alpha) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / cols8, c = (i - r * cols8) * 8;
+    float g[8], u[8];
+    ld8(gate + r * stride + c, g);
+    ld8(up + r * stride + c, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gc = fminf(g[e], limit), uc = fminf(fmaxf(u[e], -limit), limit);
+      g[e] = gc * sigmoid_exact(alpha * gc) * (uc + 1.0f);
+    }
+    st8(out + i * 8, g);
   }
 }
 
@@ -134,7 +279,15 @@ extern "C" void seq_launch_sandwich_residual(float* x, const void* a, const void
                                              void* out, int T_, int W, float eps, int is_f32,
                                              hipStream_t st) {
   const size_t lds = (size_t)W * sizeof(float);
-  if (b != nullptr) {
+  const bool v8 = W % 8 == 0 && aligned16(x) && aligned16(a) && aligned16(b) && aligned16(out) &&
+                  aligned16(wa) && aligned16(wb) && aligned16(w_post) && aligned16(w_next);
+  if (v8 && b != nullptr) {
+    DISPATCH_T(is_f32, hipLaunchKernelGGL((sandwich_residual_v8_kernel<T, true>), dim3(T_), dim3(256), lds, st,
+                                          x, (const T*)a, (const T*)b, wa, wb, w_post, w_next, (T*)out, W, eps);)
+  } else if (v8) {
+    DISPATCH_T(is_f32, hipLaunchKernelGGL((sandwich_residual_v8_kernel<T, false>), dim3(T_), dim3(256), lds, st,
+                                          x, (const T*)a, (const T*)b, wa, wb, w_post, w_next, (T*)out, W, eps);)
+  } else if (b != nullptr) {
     DISPATCH_T(is_f32, hipLaunchKernelGGL((sandwich_residual_kernel<T, true>), dim3(T_), dim3(256), lds, st,
                                           x, (const T*)a, (const T*)b, wa, wb, w_post, w_next, (T*)out, W, eps);)
   } else {
@@ -146,6 +299,23 @@ extern "C" void seq_launch_sandwich_residual(float* x, const void* a, const void
 extern "C" void seq_launch_gated_rmsnorm(void* out, const float* o, const float* w, const void* gate,
                                          int T_, int G, int S, int gate_stride, float eps, int is_f32,
                                          hipStream_t st) {
+  if (S % 8 == 0 && gate_stride % 8 == 0 && aligned16(out) && aligned16(o) && aligned16(w) && aligned16(gate)) {
+    const int lpg = S / 8;
+    if (lpg <= 64 && (lpg & (lpg - 1)) == 0) {
+      const int64_t rows = (int64_t)T_ * G;
+      const int grid = (int)((rows * lpg + 255) / 256);
+      DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_rows_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
+                                            o, w, (const T*)gate, rows, G, S, lpg, gate_stride, eps);)
+      return;
+    }
+    int threads = ((lpg + 1) / 2 + WAVE - 1) / WAVE * WAVE;       // two chunks of 8 per thread
+    if (threads <= 1024) {
+      if (threads < WAVE) threads = WAVE;
+      DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_v8_kernel<T>, dim3(T_, G), dim3(threads), 0, st,
+                                            (T*)out, o, w, (const T*)gate, S, gate_stride, eps);)
+      return;
+    }
+  }
   const int threads = S >= 256 ? 256 : (S > 64 ? 128 : 64);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_, G), dim3(threads), 0, st, (T*)out,
                                         o, w, (const T*)gate, S, gate_stride, eps);)
@@ -153,6 +323,13 @@ extern "C" void seq_launch_gated_rmsnorm(void* out, const float* o, const float*
 
 extern "C" void seq_launch_clamped_glu(void* out, const void* gate, const void* up, int64_t rows, int cols,
                                        int stride, float limit, float alpha, int is_f32, hipStream_t st) {
+  if (cols % 8 == 0 && stride % 8 == 0 && aligned16(out) && aligned16(gate) && aligned16(up)) {
+    const int64_t n8 = rows * cols / 8;
+    const int g8 = (int)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(clamped_glu_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)out,
+                                          (const T*)gate, (const T*)up, n8, cols / 8, stride, limit, alpha);)
+    return;
+  }
   const int64_t n = rows * cols;
   const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(clamped_glu_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,

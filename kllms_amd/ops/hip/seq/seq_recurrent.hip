@@ -42,6 +42,29 @@ __global__ void linear_prep_kernel(float* __restrict__ pk, const T* __restrict__
   }
 }
 
+// 8-wide form: D, V and the strides are multiples of 8, so a group of 8
+// never straddles q | k | v
+template <typename T>
+__global__ void linear_prep_v8_kernel(float* __restrict__ pk, const T* __restrict__ q,
+                                      const T* __restrict__ k, const T* __restrict__ v, int64_t n8, int H,
+                                      int D, int V, int q_stride, int k_stride, int v_stride) {
+  const int W8 = (2 * D + V) / 8;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t th = i / W8;
+    const int c = (int)(i - th * W8) * 8;
+    const int64_t t = th / H;
+    const int h = (int)(th - t * H);
+    float x[8];
+    if (c < D) ld8(q + t * q_stride + (int64_t)h * D + c, x);
+    else if (c < 2 * D) ld8(k + t * k_stride + (int64_t)h * D + (c - D), x);
+    else ld8(v + t * v_stride + (int64_t)h * V + (c - 2 * D), x);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = silu_exact(x[e]);
+    st8(pk + i * 8, x);
+  }
+}
+
 template <int DMAX, int NS>
 __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
     float* __restrict__ o, const float* __restrict__ pk, const float* __restrict__ decay,
@@ -122,7 +145,8 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
 }
 
 // ---- short causal convolution + silu ----------------------------------------
-// y[t,c] = silu(sum_j w[c,j] * x[t - (K-1-j), c]); inputs before the segment
+// y[t,c] = silu(sum_j w[j,c] * x[t - (K-1-j), c]) (weights taps-major [K, C],
+// last tap = current token); inputs before the segment
 // come from conv_state [slot, K-1, C] (oldest first), zeros for a fresh sequence.
 template <typename T>
 __global__ void causal_conv_silu_kernel(T* __restrict__ y, const T* __restrict__ x,
@@ -143,9 +167,42 @@ __global__ void causal_conv_silu_kernel(T* __restrict__ y, const T* __restrict__
       float xv;
       if (src >= 0) xv = ldf(x + (int64_t)(t - (K - 1 - j)) * x_stride + c);
       else xv = fresh ? 0.f : ldf(hist + (int64_t)(K - 1 + src) * C + c);
-      acc += w[(int64_t)c * K + j] * xv;
+      acc += w[(int64_t)j * C + c] * xv;
     }
     stf(y + idx, silu_exact(acc));
+  }
+}
+
+// 8 channels per thread (C and the row stride multiples of 8)
+template <typename T>
+__global__ void causal_conv_silu_v8_kernel(T* __restrict__ y, const T* __restrict__ x,
+                                           const float* __restrict__ w, const T* __restrict__ conv_state,
+                                           const int* __restrict__ slots, const int* __restrict__ cu,
+                                           const int* __restrict__ seg_start,
+                                           const int* __restrict__ token_seg, int64_t n8, int C, int K,
+                                           int x_stride) {
+  const int C8 = C / 8;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n8;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int t = (int)(idx / C8), c = (int)(idx - (int64_t)t * C8) * 8;
+    const int b = token_seg[t];
+    const int i = t - cu[b];
+    const bool fresh = seg_start[b] == 0;
+    const T* hist = conv_state + (int64_t)slots[b] * (K - 1) * C;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < K; ++j) {
+      const int src = i - (K - 1 - j);
+      float xv[8], wv[8];
+      if (src >= 0) ld8(x + (int64_t)(t - (K - 1 - j)) * x_stride + c, xv);
+      else if (!fresh) ld8(hist + (int64_t)(K - 1 + src) * C + c, xv);
+      else continue;
+      ld8(w + (int64_t)j * C + c, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += wv[e] * xv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = silu_exact(acc[e]);
+    st8(y + (int64_t)t * C + c, acc);
   }
 }
 
@@ -342,9 +399,17 @@ extern "C" void seq_launch_linear_attn_decay(float* o, const void* q, const void
                                              int v_stride, int is_f32, hipStream_t st) {
   const int64_t n = (int64_t)T_ * H * (2 * D + V);
   const int grid = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
-  DISPATCH_T(is_f32, hipLaunchKernelGGL(linear_prep_kernel<T>, dim3(grid), dim3(256), 0, st, packed,
-                                        (const T*)q, (const T*)k, (const T*)v, n, H, D, V, q_stride, k_stride,
-                                        v_stride);)
+  if (D % 8 == 0 && V % 8 == 0 && q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 &&
+      aligned16(q) && aligned16(k) && aligned16(v) && aligned16(packed)) {
+    const int g8 = (int)((n / 8 + 255) / 256 < 16384 ? (n / 8 + 255) / 256 : 16384);
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(linear_prep_v8_kernel<T>, dim3(g8), dim3(256), 0, st, packed,
+                                          (const T*)q, (const T*)k, (const T*)v, n / 8, H, D, V, q_stride,
+                                          k_stride, v_stride);)
+  } else {
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(linear_prep_kernel<T>, dim3(grid), dim3(256), 0, st, packed,
+                                          (const T*)q, (const T*)k, (const T*)v, n, H, D, V, q_stride, k_stride,
+                                          v_stride);)
+  }
   const int ns = pick_split(B, H, V);
   DISPATCH_NS(ns, DISPATCH_D(D, hipLaunchKernelGGL((linear_attn_decay_kernel<DMAX, NS>),
                                                    dim3(B, H, (V + WAVE / NS - 1) / (WAVE / NS)), dim3(WAVE), 0,
@@ -358,8 +423,14 @@ extern "C" void seq_launch_causal_conv_silu(void* y, const void* x, const float*
   const int64_t n = (int64_t)T_ * C;
   const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   const int grid2 = (int)(((int64_t)B * C + 255) / 256);
+  const bool v8 = C % 8 == 0 && x_stride % 8 == 0 && aligned16(y) && aligned16(x) && aligned16(conv_state) &&
+                  aligned16(w);
+  const int g8 = (int)((n / 8 + 255) / 256 < 16384 ? (n / 8 + 255) / 256 : 16384);
   DISPATCH_T(is_f32,
-             hipLaunchKernelGGL(causal_conv_silu_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)y, (const T*)x,
+             if (v8) hipLaunchKernelGGL(causal_conv_silu_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)y,
+                                        (const T*)x, w, (const T*)conv_state, slots, cu, seg_start, token_seg,
+                                        n / 8, C, K, x_stride);
+             else hipLaunchKernelGGL(causal_conv_silu_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)y, (const T*)x,
                                 w, (const T*)conv_state, slots, cu, seg_start, token_seg, n, C, K, x_stride);
              hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(grid2), dim3(256), 0, st, (const T*)x,
                                 (T*)conv_state, slots, cu, seg_start, B, C, K, x_stride);)

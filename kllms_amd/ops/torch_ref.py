@@ -388,11 +388,11 @@ def gated_rmsnorm(o, weight, gate, eps, out_dtype) -> torch.Tensor:
 
 
 def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
-    """Per-channel causal convolution over time + silu. x [T,C]; w [C,K] (last
-    column = current token); conv_state [slots, K-1, C] holds each sequence's
-    last K-1 inputs (oldest first) and is updated."""
+    """Per-channel causal convolution over time + silu. x [T,C]; w [K,C]
+    taps-major (last row = current token); conv_state [slots, K-1, C] holds
+    each sequence's last K-1 inputs (oldest first) and is updated."""
     T, C = x.shape
-    K = w.shape[1]
+    K = w.shape[0]
     y = torch.empty(T, C, dtype=x.dtype, device=x.device)
     cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
     wf = w.float()
@@ -402,7 +402,7 @@ def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start) -> to
         ext = torch.cat([hist, x[s:e].float()], 0)           # [K-1+L, C]
         acc = torch.zeros(e - s, C, device=x.device)
         for j in range(K):
-            acc += ext[j:j + (e - s)] * wf[:, j]
+            acc += ext[j:j + (e - s)] * wf[j]
         y[s:e] = torch.nn.functional.silu(acc).to(x.dtype)
         conv_state[sl[b]] = ext[ext.shape[0] - (K - 1):].to(conv_state.dtype)
     return y

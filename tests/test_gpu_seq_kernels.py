@@ -61,8 +61,9 @@ def test_embed_and_norms(dtype, W):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dual", [False, True])
 @pytest.mark.parametrize("nxt", [False, True])
-def test_sandwich_residual(dtype, dual, nxt):
-    T, W = 9, 328
+@pytest.mark.parametrize("W", [328, 36])      # 8-wide path / scalar path
+def test_sandwich_residual(dtype, dual, nxt, W):
+    T = 9
     x = rnd(T, W, std=3.0)
     a, b = rnd(T, W, dtype=dtype, seed=1), rnd(T, W, dtype=dtype, seed=2)
     wa, wb, wp, wn = (rnd(W, seed=s) * 0.2 + 1 for s in (3, 4, 5, 6))
@@ -78,16 +79,17 @@ def test_sandwich_residual(dtype, dual, nxt):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_gated_rmsnorm_and_glu(dtype):
-    T, G, S = 7, 3, 72
+@pytest.mark.parametrize("S,off,ff", [(72, 8, 104), (70, 3, 101), (128, 16, 96), (4096, 0, 64)])   # 8-wide / scalar / short-row / long-row
+def test_gated_rmsnorm_and_glu(dtype, S, off, ff):
+    T, G = 7, 3
     o = rnd(T, G, S, std=2.0)
     w = rnd(S) * 0.1 + 1
     fused = rnd(T, G * S + 24, dtype=dtype, seed=3)
-    gate = fused[:, 8:8 + G * S]
+    gate = fused[:, off:off + G * S]
     close(ops.gated_rmsnorm(o, w, gate, 1e-6, dtype), torch_ref.gated_rmsnorm(o, w, gate, 1e-6, dtype), dtype)
-    gu = rnd(T, 2 * 104, dtype=dtype, std=2.0, seed=5)
-    close(ops.clamped_glu(gu[:, :104], gu[:, 104:], 1.5, 1.702),
-          torch_ref.clamped_glu(gu[:, :104], gu[:, 104:], 1.5, 1.702), dtype)
+    gu = rnd(T, 2 * ff, dtype=dtype, std=2.0, seed=5)
+    close(ops.clamped_glu(gu[:, :ff], gu[:, ff:], 1.5, 1.702),
+          torch_ref.clamped_glu(gu[:, :ff], gu[:, ff:], 1.5, 1.702), dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -127,7 +129,7 @@ def test_rope_store_and_blocklocal_attention(dtype, D, R, mask):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,V", [(3, 24, 40), (2, 64, 130), (1, 128, 64)])
+@pytest.mark.parametrize("H,D,V", [(3, 24, 40), (2, 64, 130), (1, 128, 64), (3, 20, 33)])
 def test_linear_attn_decay(dtype, H, D, V):
     lens, starts = [33, 1, 5], [0, 9, 2]
     T = sum(lens)
@@ -145,15 +147,15 @@ def test_linear_attn_decay(dtype, H, D, V):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("K", [2, 4, 7])
-def test_causal_conv_silu(dtype, K):
-    C = 88
+@pytest.mark.parametrize("C,off", [(88, 8), (84, 5)])      # 8-wide path / scalar path
+def test_causal_conv_silu(dtype, K, C, off):
     lens, starts = [20, 1, 2, 3], [0, 5, 1, 0]
     T = sum(lens)
     cu, st, tseg = segments(lens, starts)
     slots = torch.tensor([3, 1, 0, 2], dtype=torch.int32, device=DEV)
     fused = rnd(T, C + 16, dtype=dtype, seed=1)
-    x = fused[:, 8:8 + C]
-    w = rnd(C, K, seed=2) * 0.5
+    x = fused[:, off:off + C]
+    w = rnd(K, C, seed=2) * 0.5
     hist = rnd(4, K - 1, C, dtype=dtype, seed=3)
     h1, h2 = hist.clone(), hist.clone()
     y1 = ops.causal_conv_silu(x, w, h1, slots, cu, st, tseg)
