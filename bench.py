@@ -127,7 +127,7 @@ def make_schema():
     bounds (maxLength / maxItems / integer ranges) so the byte DFA forces
     structurally complete objects in a bounded token budget — on random-init
     weights an unbounded field would run to the max_tokens cap instead of
-    closing (the round-1 schema_valid caveat)."""
+    closing (an earlier schema_valid caveat)."""
     from typing import List
 
     from pydantic import BaseModel, Field

@@ -1,6 +1,6 @@
 """On-device consensus acceleration (M5).
 
-The alignment hot loop (SURVEY §3.4) evaluates O(L^2 * m^2) pairwise
+The alignment hot loop evaluates O(L^2 * m^2) pairwise
 similarities; with the "embeddings" method each NEW long-string pair costs an
 embedding computation in the reference — one remote API roundtrip per string
 (consensus_utils.py:652-657). Locally the same contract is served in ONE

@@ -4,8 +4,8 @@ The reference duplicates the entire consensus engine as line-for-line async
 mirrors (ref consensus_utils.py:1523-2274, consolidation.py:219-303,402-493).
 Here the async API is a thin bridge over the one shared sync implementation:
 the consensus math runs in a worker thread (it is pure CPU/GPU compute with no
-awaits in the reference either — its async mirror is sequential awaits, SURVEY
-§3.3), and the caller's *async* embedding callable is bridged back onto the
+awaits in the reference either — its async mirror is sequential awaits),
+and the caller's *async* embedding callable is bridged back onto the
 running event loop via run_coroutine_threadsafe. Observable semantics are
 identical to the reference mirrors.
 """

@@ -1,7 +1,7 @@
 """Consolidation layer: n ChatCompletion choices -> one consensus completion.
 
 Behavioral re-implementation of k_llms/utils/consolidation.py:25-493.
-Invariants (ref consolidation.py:116-144):
+Invariants (ref consolidation.py:116-144.1):
 - ``len(choices) == n+1``; ``choices[0]`` is the consensus;
 - ``choices[i].index == i``; originals keep their own finish_reason/logprobs;
 - consensus choice borrows finish_reason/logprobs/function_call/tool_calls/

@@ -73,7 +73,7 @@ class LocalEngineClient:
         self.chat = _ChatNS(self)
         self.beta = _BetaNS(self)
         self.embeddings = _EmbeddingsNS(self)
-        # model used by the llm string-consensus mode (SURVEY C34): the local
+        # model used by the llm string-consensus mode: the local
         # serving model itself.
         self.consensus_model = self.config.model
 
@@ -314,8 +314,7 @@ class LocalEngineClient:
         return ChoiceLogprobs(content=toks)
 
     def _mk_timings(self, out) -> Dict[str, Any]:
-        """Per-request serving metrics (tokens/s, per-phase wall
-        times) attached as an extra `timings` field on the response."""
+        """Per-request serving metrics attached as an extra `timings` field on the response."""
         tm = dict(getattr(self.engine, "last_timings", {}))
         completion_tokens = sum(len(s.token_ids) for s in out.streams)
         decode_s = tm.get("decode_ms", 0.0) / 1000.0
@@ -331,7 +330,7 @@ class LocalEngineClient:
     def _mk_usage(self, out) -> CompletionUsage:
         completion_tokens = sum(len(s.token_ids) for s in out.streams)
         # prompt charged once for n>1 — shared prefill (OpenAI-matching
-        # semantics)
+        # semantics.5)
         return CompletionUsage(
             prompt_tokens=out.prompt_tokens,
             completion_tokens=completion_tokens,

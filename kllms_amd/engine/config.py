@@ -1,6 +1,6 @@
 """Engine and model-architecture configuration.
 
-The reference has a default-only consensus config (SURVEY §5.6); the native
+The reference has a default-only consensus config; the native
 engine adds EngineConfig — model preset/path, dtype, TP degree, KV block
 size, hipGraph toggle — exposed through ``KLLMs(**kwargs)``.
 

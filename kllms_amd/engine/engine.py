@@ -6,7 +6,7 @@ One ``generate()`` call takes a batch of requests, prefills every prompt ONCE
 in a packed varlen batch, forks each prompt's KV blocks n ways (copy-on-write
 paged cache), and steps all decode streams together until completion.
 
-Usage semantics mirror OpenAI's n>1 accounting (SURVEY §5.5): prompt tokens
+Usage semantics mirror OpenAI's n>1 accounting: prompt tokens
 counted once per request (the prefill is genuinely shared), completion tokens
 summed across the n streams.
 """
@@ -56,7 +56,7 @@ class StreamOutput:
 class RequestOutput:
     prompt_tokens: int
     streams: List[StreamOutput] = field(default_factory=list)
-    # wall-clock phase timings (observability)
+    # wall-clock phase timings (observability.1)
     prefill_ms: float = 0.0
     decode_ms: float = 0.0
 
@@ -151,7 +151,7 @@ class LLMEngine:
             self.ctx = ParallelContext()
 
         # size-switched custom collective: one-shot xGMI all-reduce for small
-        # (decode-step) tensors, RCCL ring above threshold (SURVEY §5.8)
+        # (decode-step) tensors, RCCL ring above threshold
         if self.ctx.world_size > 1 and self.ctx.custom_ar is None:
             from ..parallel.collective import maybe_init_custom_allreduce
 
@@ -942,7 +942,7 @@ class LLMEngine:
         mode = getattr(self.config, "embedding_mode", "auto")
         if mode != "auto":
             return mode
-        # random-init token embeddings are semantic noise (VERDICT r1 item 5);
+        # random-init token embeddings are semantic noise;
         # the signed n-gram hash tracks string similarity with no weights
         return "token_mean" if self.config.effective_weights_dir() else "ngram"
 
@@ -984,7 +984,7 @@ class LLMEngine:
         """Device-resident variant of embed(): returns the [N, H] float32
         unit-vector tensor ON the engine device (zero rows for empty texts),
         so the consensus accel can run its cosine GEMM without a host round
-        trip (consolidation similarity math on-device)."""
+        trip."""
         if self._embedding_mode() == "ngram":
             return self._embed_ngram_dev(texts)
         emb = self.model.embed_tokens.weight

@@ -350,7 +350,7 @@ class HybridStateCache(PagedKVCache):
 
 
 class PrefixCache:
-    """Shared-prefix KV reuse across requests (VERDICT r1 item 8).
+    """Shared-prefix KV reuse across requests.
 
     Consensus batches share the chat-template header, and real serving
     usually shares a long system prompt; this maps a chain digest of each

@@ -1,6 +1,6 @@
 """Safetensors weight loading with per-TP-rank sharding.
 
-The load-only "checkpoint" subsystem (SURVEY §5.4): maps HuggingFace-style
+The load-only "checkpoint" subsystem: maps HuggingFace-style
 Llama/Mixtral parameter names onto this model's fused/sharded layout and
 slices each rank's shard while streaming tensors from the safetensors files
 (no full-model host copy).

@@ -168,7 +168,7 @@ class LlamaForCausalLM(nn.Module):
         self.norm = RMSNormModule(cfg.hidden_size, cfg.rms_norm_eps, dtype)
         # LM head replicated across TP ranks: hidden states are replicated
         # after each layer's all-reduce, so full logits come out identical on
-        # every rank — no logits gather needed (SURVEY §2.3 point 3).
+        # every rank — no logits gather needed.
         self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False, dtype=dtype)
         self.lm_head.weight.requires_grad_(False)
         self.register_buffer(

@@ -3,8 +3,7 @@
 Same attention/backbone as Llama (GQA, RoPE, RMSNorm); the MLP is a
 top-k-routed mixture of experts. Experts are TP-SHARDED, not
 expert-parallel — every rank holds a 1/tp slice of every expert, so routing
-needs no all-to-all and the layer keeps the dense model's two all-reduces
-("experts TP-sharded so no all-to-all").
+needs no all-to-all and the layer keeps the dense model's two all-reduces.
 
 Expert compute has two regimes: decode shapes run a DENSE batched GEMM over
 all experts (same HBM traffic as routed compute when nearly every expert is
@@ -89,7 +88,7 @@ class MixtralMoE(nn.Module):
         (ops/hip/moe.hip) over tokens sorted by expert — gate/up GEMM with
         fused silu*mul, then the down GEMM — plus one index_add to scatter
         the routing-weighted rows back to token order. Replaces the
-        per-expert loop (<=2 GEMM launches per layer)."""
+        per-expert loop."""
         from .. import ops
 
         BM = 128

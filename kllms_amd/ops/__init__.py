@@ -1,6 +1,6 @@
 """Op dispatch: HIP/CDNA4 kernels on GPU, torch reference on CPU.
 
-Policy (BASELINE north star): on a GPU (`tensor.is_cuda`, which on
+Policy: on a GPU (`tensor.is_cuda`, which on
 PyTorch-ROCm means an AMD GPU) the hand-written gfx950 HIP kernels in
 ``kllms_amd._C`` are the ONLY path — if the extension is missing the op
 RAISES instead of silently falling back to eager PyTorch. On CPU the pure

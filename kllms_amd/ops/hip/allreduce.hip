@@ -1,7 +1,7 @@
 // One-shot all-reduce for small (latency-bound) decode-step tensors, over
 // hipIpc-mapped peer buffers on the xGMI mesh.
 //
-// SURVEY §5.8 / §2.3: on an 8-GPU MI355X node the xGMI fabric is fully
+// on an 8-GPU MI355X node the xGMI fabric is fully
 // connected (7 p2p links per GPU), so for the tens-of-KB tensors a TP decode
 // step reduces ([n_streams, hidden] bf16) the latency-optimal schedule is
 // ONE SHOT: every rank reads all peers' staged buffers directly over xGMI
@@ -16,8 +16,8 @@
 //   2. after the reduce: same handshake on end[block][*] — guarantees no
 //      rank re-stages its buffer while a peer is still reading it.
 // Epochs come from a DEVICE-resident per-block counter, so the kernel is
-// hipGraph-replayable (no per-launch salt argument — frozen under replay;
-// cdna_hip_programming.md §6 G16 "Re-initialise every call").
+// hipGraph-replayable (no per-launch salt argument — it would be frozen
+// under replay).
 // Spins are BOUNDED: a dead peer trips s_trap instead of hanging the GPU.
 //
 // Reference parity note: the reference has no collectives (its backend is a

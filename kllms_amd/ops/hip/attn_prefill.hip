@@ -1,6 +1,6 @@
 // Varlen causal prefill attention for gfx950 — flash-style MFMA kernel.
 //
-// Structure (cdna_hip_programming.md Appendix B "Fused attention prefill"):
+// Structure:
 //   - an 8-WAVE workgroup serves 8 consecutive 32-row q-tiles of ONE
 //     (sequence, q-head): the K/V LDS staging is shared by the 8 waves, so
 //     its cost is amortized 8x over the 1-wave-per-block version;

@@ -1,6 +1,6 @@
 // Batched Levenshtein distance for the on-device consensus path (gfx950).
 //
-// SURVEY §5.8 / VERDICT r1 item 9: the consolidator's string-similarity
+// the consolidator's string-similarity
 // matrices should run on-device. Long (>50 char) strings already go through
 // the batched embedding + cosine GEMM path (consensus/accel.py); this kernel
 // covers the SHORT pairs, which the reference scores with normalized

@@ -1,6 +1,6 @@
 // Grouped MoE expert GEMMs for gfx950 (Mixtral prefill path).
 //
-// VERDICT r1 item 5: replace the per-expert Python loop (8 experts x
+// replace the per-expert Python loop (8 experts x
 // mask/gather/2 GEMM/index_add per layer) with TWO MFMA kernel launches:
 //
 //   moe_gateup_kernel: act[s, :] = silu(x[tok(s)] @ Wg[e]^T) * (x[tok(s)] @ Wu[e]^T)

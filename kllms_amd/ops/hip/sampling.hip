@@ -12,8 +12,7 @@
 //           only the boundary bin at 256x finer resolution each time —
 //           threshold resolution 20/256^4 ~ 5e-9 in scaled-logit space, i.e.
 //           exact top-k/top-p up to fp32 rounding of the logits themselves
-//           (the old single-pass cut admitted everything
-//           within one 0.078-wide bin of the true boundary)
+//
 //   pass D: Gumbel-max draw over admitted tokens — counter-based RNG
 //           hash(seed, step, token): deterministic, stream-ordered, and
 //           identical regardless of batch composition.

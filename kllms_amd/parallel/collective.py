@@ -1,6 +1,6 @@
 """Size-switched TP collective: custom one-shot xGMI all-reduce + RCCL ring.
 
-SURVEY §5.8: decode-step tensors ([n_streams, hidden] bf16, tens of KB) are
+decode-step tensors ([n_streams, hidden] bf16, tens of KB) are
 LATENCY-bound on the fully-connected xGMI mesh — every rank reads all peers
 directly (one hop) instead of paying the ring's 2(N-1) hops. Prefill
 activations (MBs) are BANDWIDTH-bound — the RCCL ring saturates the per-link

@@ -1,7 +1,7 @@
 """Tensor parallelism over RCCL / xGMI.
 
 The reference has zero distributed code (its backend is a remote API); this is
-the native sharding layer the BASELINE configs require (SURVEY §2.2, §2.3):
+the native sharding layer the BASELINE configs require:
 column/row-parallel linear layers with an all-reduce after the attention
 output projection and the MLP down projection — exactly 2 all-reduces per
 transformer layer at TP > 1.

@@ -1,4 +1,4 @@
-"""hipIpc one-shot all-reduce on real hardware (VERDICT round-1 item 1).
+"""hipIpc one-shot all-reduce on real hardware.
 
 A gpurun box has ONE MI355X, so multi-rank validation runs as 2 processes
 SHARING cuda:0: hipIpc handle exchange, the two-phase epoch handshake and the

@@ -551,7 +551,7 @@ class TestOneShotAllreduce:
     def test_allreduce_matches_fp32_sum(self):
         """One-shot all-reduce (single-GPU peer simulation): all N buffers end
         holding the fp32-accumulated sum of the inputs (round-2 groundwork
-        for the xGMI one-shot path)."""
+        for the xGMI one-shot path.3/§5.8)."""
         from kllms_amd import ops as kops
 
         torch.manual_seed(5)
@@ -574,7 +574,7 @@ class TestOneShotAllreduce:
 
 class TestMoEGroupedGEMM:
     """Grouped MoE MFMA kernels (ops/hip/moe.hip) vs the per-expert torch
-    loop on identical routing — VERDICT r1 item 5."""
+    loop on identical routing."""
 
     def _moe(self, E=8, I=512, H=512, k=2, seed=0):
         from kllms_amd.engine.config import ModelArchConfig

@@ -1,4 +1,4 @@
-"""Cross-request prefix caching (kvcache.PrefixCache; VERDICT r1 item 8).
+"""Cross-request prefix caching (kvcache.PrefixCache).
 
 Correctness bar: a prefix-cache hit must be OUTPUT-INVISIBLE — identical
 greedy tokens and logprobs vs an engine with caching disabled — while

@@ -1,5 +1,5 @@
 """Tokenizer tests: byte-level round trips, chat templating, crop semantics
-(the local equivalents of the reference's tiktoken usage)."""
+(the local equivalents of the reference's tiktoken usage.2)."""
 
 import os
 import pytest

@@ -1,7 +1,7 @@
 """Tensor-parallel correctness over torch.distributed (gloo, world_size=2).
 
 The distributed path must be correct by construction before it ever touches
-an 8-GPU node (SURVEY §4 item 4): TP=2 over gloo on CPU must reproduce the
+an 8-GPU node: TP=2 over gloo on CPU must reproduce the
 TP=1 model's logits (the random init is TP-degree-invariant by design), and
 the engine must produce identical greedy decodes on every rank.
 """

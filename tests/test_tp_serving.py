@@ -1,6 +1,6 @@
 """TP>1 serving over the continuous-batching scheduler (gloo, world_size=2).
 
-VERDICT round-1 item 2: the scheduler must serve TP>1 — rank 0 broadcasts
+the scheduler must serve TP>1 — rank 0 broadcasts
 every engine-touching phase (admit / chunked-prefill advance / decode step)
 and the follower ranks replay them in lockstep (kllms_amd/parallel/serve.py).
 Covers: plain create, n>1 fan-out, constrained (parse) requests crossing the
