@@ -137,6 +137,93 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
   }
 }
 
+// The same attention with coalesced 8-wide accesses — the decode kernel (and
+// the one for continuing rows of a prompt portion). Needs D and Dv multiples
+// of 8 with D/8 and Dv/8 powers of two <= 64, 16-byte aligned rows.
+//   scores: LPK = D/8 lanes share one key (each holds 8 dims of q in registers
+//           and loads 16 B of the key row), 64/LPK keys per pass, the partial
+//           dots are summed inside the lane group;
+//   values: LPV = Dv/8 lanes share one key's value row, 64/LPV keys per pass,
+//           each lane accumulates 8 output dims; the key groups are summed
+//           once at the end.
+// Tiles of 64 keys, online softmax in fp32 as above.
+template <typename T>
+__global__ void __launch_bounds__(WAVE) attn_blocklocal_paged_v8_kernel(
+    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, const int* __restrict__ token_seg,
+    const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
+    float scale, int mask_size, int H, int G, int D, int Dv, int BS, int bt_stride, int q_stride,
+    int gate_stride) {
+  __shared__ float ps[WAVE];
+  __shared__ int rows[WAVE];
+  const int t = row_map ? row_map[blockIdx.x] : blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (H / G);
+  const int p = (int)positions[t];
+  const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
+  const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
+  const int LPK = D / 8, KPI = WAVE / LPK, kpart = lane % LPK, kgrp = lane / LPK;
+  const int LPV = Dv / 8, KPV = WAVE / LPV, vpart = lane % LPV, vgrp = lane / LPV;
+  float qv[8];
+  ld8(q + (int64_t)t * q_stride + (int64_t)h * D + kpart * 8, qv);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) qv[e] *= scale;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  for (int base = lo; base <= p; base += WAVE) {
+    const int n = min(WAVE, p - base + 1);
+    const int j = base + lane;
+    rows[lane] = j <= p ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
+    __syncthreads();
+    for (int it = 0; it * KPI < n; ++it) {
+      const int key = it * KPI + kgrp;
+      float d = 0.f;
+      if (key < n) {
+        float kv[8];
+        ld8(k_cache + (int64_t)rows[key] * D + kpart * 8, kv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d += qv[e] * kv[e];
+      }
+      for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off);
+      if (kpart == 0 && key < n) ps[key] = d;
+    }
+    __syncthreads();
+    const float s = lane < n ? ps[lane] : -INFINITY;
+    const float m_new = fmaxf(m, wave_max(s));
+    const float w = lane < n ? expf(s - m_new) : 0.f;
+    const float corr = expf(m - m_new);        // m = -inf on the first tile -> 0
+    l = l * corr + wave_sum(w);
+    m = m_new;
+    __syncthreads();                           // every lane has read its score
+    ps[lane] = w;
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= corr;
+    for (int it = 0; it * KPV < n; ++it) {
+      const int key = it * KPV + vgrp;
+      if (key < n) {
+        float vv[8];
+        ld8(v_cache + (int64_t)rows[key] * Dv + vpart * 8, vv);
+        const float pw = ps[key];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += pw * vv[e];
+      }
+    }
+    __syncthreads();
+  }
+  for (int off = LPV; off < WAVE; off <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], off);
+  }
+  if (vgrp == 0) {
+    float gsc = 1.0f / l;
+    if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= gsc;
+    st8(out + ((int64_t)t * H + h) * Dv + vpart * 8, acc);
+  }
+}
+
 // out[t, h, :] *= sigmoid(gate[t, h]) — the per-head output gate for rows
 // whose attention came from a kernel without it
 template <typename T>
@@ -192,6 +279,15 @@ extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const
                                                  int gate_stride, int is_f32, hipStream_t st) {
   const size_t lds = (size_t)(D + 2 * WAVE) * sizeof(float);
   const int rows = row_map ? n_rows : T_;
+  const int lpk = D / 8, lpv = Dv / 8;
+  if (D % 8 == 0 && Dv % 8 == 0 && lpk <= 64 && lpv <= 64 && (lpk & (lpk - 1)) == 0 && (lpv & (lpv - 1)) == 0 &&
+      q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out)) {
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE), 0, st,
+                                          (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
+                                          block_tables, token_seg, positions, (const T*)gate, row_map, scale,
+                                          mask_size, H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
+    return;
+  }
   DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(rows, H), dim3(WAVE), lds, st,
                                         (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
                                         block_tables, token_seg, positions, (const T*)gate, row_map, scale,

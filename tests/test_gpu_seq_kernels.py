@@ -93,8 +93,9 @@ def test_gated_rmsnorm_and_glu(dtype, S, off, ff):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("D,R,mask", [(64, 32, 24), (40, 10, 0), (128, 64, 100)])
-def test_rope_store_and_blocklocal_attention(dtype, D, R, mask):
+@pytest.mark.parametrize("D,R,mask,pad", [(64, 32, 24, 8), (40, 10, 0, 6), (128, 64, 100, 8), (64, 8, 24, 6),
+                                          (16, 8, 0, 8)])      # pad 8: aligned rows (8-wide kernel); 6: scalar kernel
+def test_rope_store_and_blocklocal_attention(dtype, D, R, mask, pad):
     H, G, BS, NB = 6, 2, 16, 40
     lens, starts = [50, 1, 7, 1], [0, 130, 37, 24]
     T = sum(lens)
@@ -113,13 +114,13 @@ def test_rope_store_and_blocklocal_attention(dtype, D, R, mask):
     inv_freq = (10000.0 ** (-torch.arange(R, dtype=torch.float64) * 2 / (2 * R))).float().to(DEV)
     kc = rnd(NB, G, BS, D, dtype=dtype, seed=7)    # stands for keys stored by earlier steps
     vc = rnd(NB, G, BS, D, dtype=dtype, seed=8)
-    fused = rnd(T, H * D + G * D + H, dtype=dtype, seed=9)
+    fused = rnd(T, H * D + G * D + pad, dtype=dtype, seed=9)
     res = []
     for impl in (ops, torch_ref):
         f = fused.clone()
         q = f[:, :H * D].unflatten(1, (H, D))
         k = f[:, H * D:H * D + G * D].unflatten(1, (G, D))
-        gate = f[:, H * D + G * D:]
+        gate = f[:, H * D + G * D:H * D + G * D + H]
         k1, v1 = kc.clone(), vc.clone()
         impl.rope_pairs_store(q, k, None, pos, inv_freq, k1, v1, slots)
         out = impl.attn_blocklocal_paged(q, k1, v1, bt, tseg, pos, 0.17, mask, gate)
