@@ -146,18 +146,29 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
 //   values: LPV = Dv/8 lanes share one key's value row, 64/LPV keys per pass,
 //           each lane accumulates 8 output dims; the key groups are summed
 //           once at the end.
-// Tiles of 64 keys, online softmax in fp32 as above.
+// Tiles of 64 keys, online softmax in fp32 as above; four waves per
+// (row, head) share the tiles and merge at the end.
+#define ATTN_V8_WAVES 4
 template <typename T>
-__global__ void __launch_bounds__(WAVE) attn_blocklocal_paged_v8_kernel(
+__global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ token_seg,
     const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
     float scale, int mask_size, int H, int G, int D, int Dv, int BS, int bt_stride, int q_stride,
     int gate_stride) {
-  __shared__ float ps[WAVE];
-  __shared__ int rows[WAVE];
+  // The block's waves take the key tiles in turn (tile r*NW + wave in round
+  // r), each with its own running max / sum / accumulator; the partial
+  // results are merged through LDS at the end. Every wave runs every round —
+  // a wave without a tile only keeps the barriers company.
+  constexpr int NW = ATTN_V8_WAVES;
+  __shared__ float ps_[NW][WAVE];
+  __shared__ int rows_[NW][WAVE];
+  __shared__ float part_m[NW], part_l[NW];
+  __shared__ float part_acc[NW][512];
   const int t = row_map ? row_map[blockIdx.x] : blockIdx.x;
-  const int h = blockIdx.y, lane = threadIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  float* ps = ps_[wave];
+  int* rows = rows_[wave];
   const int g = h / (H / G);
   const int p = (int)positions[t];
   const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
@@ -170,10 +181,12 @@ __global__ void __launch_bounds__(WAVE) attn_blocklocal_paged_v8_kernel(
   for (int e = 0; e < 8; ++e) qv[e] *= scale;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  for (int base = lo; base <= p; base += WAVE) {
-    const int n = min(WAVE, p - base + 1);
+  const int ntiles = (p - lo) / WAVE + 1;
+  for (int r = 0; r * NW < ntiles; ++r) {
+    const int base = lo + (r * NW + wave) * WAVE;
+    const int n = min(WAVE, p - base + 1);            // <= 0: no tile for this wave in this round
     const int j = base + lane;
-    rows[lane] = j <= p ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
+    rows[lane] = (n > 0 && j <= p) ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
     __syncthreads();
     for (int it = 0; it * KPI < n; ++it) {
       const int key = it * KPI + kgrp;
@@ -188,13 +201,16 @@ __global__ void __launch_bounds__(WAVE) attn_blocklocal_paged_v8_kernel(
       if (kpart == 0 && key < n) ps[key] = d;
     }
     __syncthreads();
-    const float s = lane < n ? ps[lane] : -INFINITY;
-    const float m_new = fmaxf(m, wave_max(s));
-    const float w = lane < n ? expf(s - m_new) : 0.f;
-    const float corr = expf(m - m_new);        // m = -inf on the first tile -> 0
-    l = l * corr + wave_sum(w);
-    m = m_new;
-    __syncthreads();                           // every lane has read its score
+    float w = 0.f, corr = 1.f;
+    if (n > 0) {                                      // uniform over the wave
+      const float s = lane < n ? ps[lane] : -INFINITY;
+      const float m_new = fmaxf(m, wave_max(s));
+      w = lane < n ? expf(s - m_new) : 0.f;
+      corr = expf(m - m_new);                         // m = -inf on the wave's first tile -> 0
+      l = l * corr + wave_sum(w);
+      m = m_new;
+    }
+    __syncthreads();                                  // every lane has read its score
     ps[lane] = w;
     __syncthreads();
 #pragma unroll
@@ -215,12 +231,30 @@ __global__ void __launch_bounds__(WAVE) attn_blocklocal_paged_v8_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], off);
   }
+  // merge the waves' partial softmaxes
+  if (lane == 0) { part_m[wave] = m; part_l[wave] = l; }
   if (vgrp == 0) {
-    float gsc = 1.0f / l;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part_acc[wave][vpart * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  if (wave == 0 && vgrp == 0) {
+    float M = part_m[0];
+#pragma unroll
+    for (int w2 = 1; w2 < NW; ++w2) M = fmaxf(M, part_m[w2]);
+    float L = 0.f, o8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) {
+      const float f = part_l[w2] > 0.f ? expf(part_m[w2] - M) : 0.f;   // a wave that saw no key
+      L += part_l[w2] * f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o8[e] += part_acc[w2][vpart * 8 + e] * f;
+    }
+    float gsc = 1.0f / L;
     if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] *= gsc;
-    st8(out + ((int64_t)t * H + h) * Dv + vpart * 8, acc);
+    for (int e = 0; e < 8; ++e) o8[e] *= gsc;
+    st8(out + ((int64_t)t * H + h) * Dv + vpart * 8, o8);
   }
 }
 
@@ -282,7 +316,7 @@ extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const
   const int lpk = D / 8, lpv = Dv / 8;
   if (D % 8 == 0 && Dv % 8 == 0 && lpk <= 64 && lpv <= 64 && (lpk & (lpk - 1)) == 0 && (lpv & (lpv - 1)) == 0 &&
       q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out)) {
-    DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE), 0, st,
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE * ATTN_V8_WAVES), 0, st,
                                           (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
                                           block_tables, token_seg, positions, (const T*)gate, row_map, scale,
                                           mask_size, H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
