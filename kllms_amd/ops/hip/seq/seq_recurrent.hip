@@ -379,9 +379,10 @@ __global__ void __launch_bounds__(WAVE) gated_delta_rule_kernel(
   else { constexpr int DMAX = 256; __VA_ARGS__ }
 
 // rows of the state are split over NS lane groups; more groups = more, smaller
-// waves. Take the coarsest split that still gives ~4 waves per SIMD.
+// waves with fewer registers each. Take the coarsest split that still gives
+// every SIMD (1024 of them) many waves to switch between.
 static inline int pick_split(int B, int H, int V) {
-  const int64_t want = 4096;
+  const int64_t want = 16384;
   for (int ns = 2; ns <= 8; ns *= 2)
     if ((int64_t)B * H * ((V + 64 / ns - 1) / (64 / ns)) >= want) return ns;
   return 8;
