@@ -156,9 +156,9 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
     const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
     float scale, int mask_size, int H, int G, int D, int Dv, int BS, int bt_stride, int q_stride,
     int gate_stride) {
-  // The block's waves take the key tiles in turn (tile r*NW + wave in round
+  // The block's waves take the key tiles in turn (tile r*NW + wave in pass
   // r), each with its own running max / sum / accumulator; the partial
-  // results are merged through LDS at the end. Every wave runs every round —
+  // results are merged through LDS at the end. Every wave runs every pass —
   // a wave without a tile only keeps the barriers company.
   constexpr int NW = ATTN_V8_WAVES;
   __shared__ float ps_[NW][WAVE];
@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
   const int ntiles = (p - lo) / WAVE + 1;
   for (int r = 0; r * NW < ntiles; ++r) {
     const int base = lo + (r * NW + wave) * WAVE;
-    const int n = min(WAVE, p - base + 1);            // <= 0: no tile for this wave in this round
+    const int n = min(WAVE, p - base + 1);            // <= 0: no tile for this wave in this pass
     const int j = base + lane;
     rows[lane] = (n > 0 && j <= p) ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
     __syncthreads();
