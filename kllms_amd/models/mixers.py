@@ -59,7 +59,12 @@ class FusedInput(nn.Module):
     """Several projections of the same input as ONE GEMM: the checkpoint's
     separate [out_i, in] matrices are stacked along the output dim (optionally
     with a bias that is zero where a part has none). ``parts`` keeps each
-    name's column range; ``split`` returns row views of the result."""
+    name's column range; ``split`` returns row views of the result. Every
+    part starts at a multiple of 8 columns and the total width is one too
+    (zero rows in between), so the views stay 16-byte aligned for the
+    kernels' vector loads whatever the part sizes are."""
+
+    ALIGN = 8
 
     def __init__(self, in_features: int, parts: List[Tuple[str, int]], dtype, bias_parts=()):
         super().__init__()
@@ -67,9 +72,9 @@ class FusedInput(nn.Module):
         off = 0
         for name, n in parts:
             self.parts[name] = (off, n)
-            off += n
-        self.weight = _param(off, in_features, dtype=dtype)
-        self.bias = _param(off, dtype=dtype) if bias_parts else None
+            off = (off + n + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        self.weight = nn.Parameter(torch.zeros(off, in_features, dtype=dtype), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(off, dtype=dtype), requires_grad=False) if bias_parts else None
         self.bias_parts = tuple(bias_parts)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -120,7 +125,8 @@ class BlockLocalAttention(nn.Module):
         (tile groups, row_map or None), or None when nothing goes dense."""
         sp = self.spec
         if (batch.host_segs is None or not q.is_cuda or q.dtype != torch.bfloat16
-                or sp.dim != 128 or sp.vdim != 128 or ops._force_torch()):
+                or sp.dim != 128 or sp.vdim != 128 or ops._force_torch()
+                or q.stride(0) % 8 or q.data_ptr() % 16):      # the dense kernel loads 16 bytes at a time
             return None
         key = ("blocklocal", sp.mask_size)
         if key in batch.plans:
@@ -265,9 +271,14 @@ class ChannelDeltaMixer(nn.Module):
         self.gd, self.hv = spec.kv_heads * spec.dim, spec.heads * spec.vdim
         self.inp = FusedInput(hidden, [("q", self.gd), ("k", self.gd), ("v", self.hv),
                                        ("a1", spec.decay_rank), ("g1", spec.gate_rank), ("b", spec.heads)], dtype)
-        # taps-major [K, C] over the q|k|v channels (the checkpoint's [C, K] transposed:
-        # the kernels read 8 channels of one tap at a time)
-        self.conv = _param(spec.conv, 2 * self.gd + self.hv, dtype=torch.float32)
+        # the convolution runs over the fused projection's q|k|v column range as it
+        # is laid out (alignment gaps included: zero taps there); weights are
+        # taps-major [K, C] (the checkpoint's [C, K] transposed: the kernels read 8
+        # channels of one tap at a time)
+        p = self.inp.parts
+        self.oq, self.ok, self.ov = p["q"][0], p["k"][0], p["v"][0]
+        self.cp = self.ov + self.hv
+        self.conv = nn.Parameter(torch.zeros(spec.conv, self.cp, dtype=torch.float32), requires_grad=False)
         self.a2 = _param(spec.heads * spec.dim, spec.decay_rank, dtype=dtype)
         self.g2 = _param(self.hv, spec.gate_rank, dtype=dtype)
         self.dt_bias = _param(spec.heads * spec.dim, dtype=torch.float32)
@@ -277,21 +288,20 @@ class ChannelDeltaMixer(nn.Module):
 
     def cache_spec(self) -> LayerCacheSpec:
         sp = self.spec
-        return LayerCacheSpec(rec=(sp.heads, sp.dim, sp.vdim), conv=(2 * self.gd + self.hv, sp.conv - 1))
+        return LayerCacheSpec(rec=(sp.heads, sp.dim, sp.vdim), conv=(self.cp, sp.conv - 1))
 
     def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
         sp = self.spec
         y = self.inp(h)
         s = self.inp.split
-        c = 2 * self.gd + self.hv
-        qkv = ops.causal_conv_silu(y[:, :c], self.conv, st.conv, batch.state_slots, batch.cu_seqlens,
+        qkv = ops.causal_conv_silu(y[:, :self.cp], self.conv, st.conv, batch.state_slots, batch.cu_seqlens,
                                    batch.seg_start, batch.token_seg)
         a = F.linear(s(y, "a1"), self.a2)
         gate = F.linear(s(y, "g1"), self.g2)
         o = ops.gated_delta_rule(
-            qkv[:, :self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
-            qkv[:, self.gd:2 * self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
-            qkv[:, 2 * self.gd:].unflatten(1, (sp.heads, sp.vdim)),
+            qkv[:, self.oq:self.oq + self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
+            qkv[:, self.ok:self.ok + self.gd].unflatten(1, (sp.kv_heads, sp.dim)),
+            qkv[:, self.ov:self.ov + self.hv].unflatten(1, (sp.heads, sp.vdim)),
             s(y, "b"), a, self.dt_bias, self.A_log, st.rec, batch.state_slots, batch.cu_seqlens,
             batch.seg_start)
         r = ops.gated_rmsnorm(o, self.norm, gate, self.eps, self.o_proj.dtype)
@@ -299,10 +309,10 @@ class ChannelDeltaMixer(nn.Module):
 
     def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
         m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
-        gd = self.gd
-        m[pre + "q.conv"] = self.conv.t()[:gd]
-        m[pre + "k.conv"] = self.conv.t()[gd:2 * gd]
-        m[pre + "v.conv"] = self.conv.t()[2 * gd:]
+        ct = self.conv.t()
+        m[pre + "q.conv"] = ct[self.oq:self.oq + self.gd]
+        m[pre + "k.conv"] = ct[self.ok:self.ok + self.gd]
+        m[pre + "v.conv"] = ct[self.ov:self.ov + self.hv]
         for n in ("a2", "g2", "dt_bias", "A_log", "norm"):
             m[pre + n] = getattr(self, n)
         m[pre + "o"] = self.o_proj

@@ -255,7 +255,7 @@ void causal_conv_silu(torch::Tensor y, torch::Tensor x, torch::Tensor w, torch::
   TORCH_CHECK(w.dim() == 2);
   const int T = x.size(0), C = x.size(1), K = w.size(0), B = slots.numel();
   TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.numel() == (int64_t)T * C && w.size(1) == C);
-  TORCH_CHECK(K >= 2 && K <= 16, "2..16 convolution taps supported");
+  TORCH_CHECK(K >= 1 && K <= 16, "1..16 convolution taps supported");
   TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(1) == K - 1 && conv_state.size(2) == C);
   TORCH_CHECK(token_seg.numel() == T);
   if (T == 0 || B == 0) return;

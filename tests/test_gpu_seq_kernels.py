@@ -147,7 +147,7 @@ def test_linear_attn_decay(dtype, H, D, V):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("K", [2, 4, 7])
+@pytest.mark.parametrize("K", [1, 2, 4, 7])
 @pytest.mark.parametrize("C,off", [(88, 8), (84, 5)])      # 8-wide path / scalar path
 def test_causal_conv_silu(dtype, K, C, off):
     lens, starts = [20, 1, 2, 3], [0, 5, 1, 0]

@@ -203,7 +203,7 @@ def test_block_mask_is_visible_in_the_output():
 
 
 @pytest.mark.parametrize("cuts", [[40], [30] + [1] * 10, [1, 2, 1, 3, 2, 31], [2] * 20])
-@pytest.mark.parametrize("conv", [2, 4, 6])
+@pytest.mark.parametrize("conv", [1, 2, 4, 6])
 def test_channel_delta_mixer(cuts, conv):
     layer = delta(heads=4, kv=2, dim=6, vdim=10, conv=conv)
     cfg = {"vocab": 8, "width": 24, "norm": {"eps": EPS}, "layers": [layer]}
