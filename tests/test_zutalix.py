@@ -385,7 +385,6 @@ def test_trace_replay_cli(tmp_path, model_b):
                        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
     assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
-    assert not (out / "1.f32").exists() or True
     la, lb = O.forward(cfg, w, a), O.forward(cfg, w, b)
     rd = lambda n: torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"]).copy())
     check(rd(0), la[[0, 17]])
