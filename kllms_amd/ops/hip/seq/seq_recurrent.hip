@@ -85,6 +85,31 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
 #pragma unroll
   for (int d = 0; d < DR; ++d) S[d] = (!fresh && live && d0 + d < D) ? sp[(int64_t)(d0 + d) * V] : 0.f;
   const float dec = decay[h];
+  if (t1 - t0 == 1) {
+    // decode: one row. No pipeline — stage q|k once (zeros above D), update, read out.
+    const float* row = pk + ((int64_t)t0 * H + h) * W;
+    float* buf = qk[0][0];
+    for (int i = lane; i < 2 * DMAX; i += WAVE) {
+      const int d = i < DMAX ? i : i - DMAX;
+      buf[i] = d < D ? row[i < DMAX ? d : D + d] : 0.f;
+    }
+    const float vj = live ? row[2 * D + j] : 0.f;
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll
+    for (int d = 0; d < DR; ++d) {
+      S[d] = dec * S[d] + buf[DMAX + d0 + d] * vj;
+      acc += S[d] * buf[d0 + d];
+    }
+#pragma unroll
+    for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
+    if (live) {
+      if (grp == 0) o[((int64_t)t0 * H + h) * V + j] = acc;
+#pragma unroll
+      for (int d = 0; d < DR; ++d) if (d0 + d < D) sp[(int64_t)(d0 + d) * V] = S[d];
+    }
+    return;
+  }
   // rows D..DMAX-1 of the staging buffers stay zero, so the unrolled loops
   // below run over DMAX without a bound check (a branch per row would keep
   // the LDS reads from being batched)
@@ -298,6 +323,44 @@ __global__ void __launch_bounds__(WAVE) gated_delta_rule_kernel(
   const bool fresh = seg_start[b] == 0;
 #pragma unroll
   for (int d = 0; d < DR; ++d) S[d] = (!fresh && live && d0 + d < D) ? sp[(int64_t)(d0 + d) * V] : 0.f;
+  if (t1 - t0 == 1) {
+    // decode: one row, no pipeline (see linear_attn_decay_kernel)
+    float* buf = buf_[0][0];
+    for (int i = lane; i < 3 * DMAX; i += WAVE) {
+      const int which = i / DMAX, d = i - which * DMAX;
+      float val = 0.f;
+      if (d < D)
+        val = which == 0 ? qn[((int64_t)t0 * G + g) * D + d]
+            : which == 1 ? kn[((int64_t)t0 * G + g) * D + d] : gd[((int64_t)t0 * H + h) * D + d];
+      buf[i] = val;
+    }
+    const float vj = live ? vf[((int64_t)t0 * H + h) * V + j] : 0.f;
+    const float beta = bt[(int64_t)t0 * H + h];
+    __syncthreads();
+    float pred = 0.f;
+#pragma unroll
+    for (int d = 0; d < DR; ++d) {
+      S[d] *= buf[2 * DMAX + d0 + d];
+      pred += S[d] * buf[DMAX + d0 + d];
+    }
+#pragma unroll
+    for (int off = COLS; off < WAVE; off <<= 1) pred += __shfl_xor(pred, off);
+    const float uu = beta * (vj - pred);
+    float acc = 0.f;
+#pragma unroll
+    for (int d = 0; d < DR; ++d) {
+      S[d] += buf[DMAX + d0 + d] * uu;
+      acc += S[d] * buf[d0 + d];
+    }
+#pragma unroll
+    for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
+    if (live) {
+      if (grp == 0) o[((int64_t)t0 * H + h) * V + j] = acc;
+#pragma unroll
+      for (int d = 0; d < DR; ++d) if (d0 + d < D) sp[(int64_t)(d0 + d) * V] = S[d];
+    }
+    return;
+  }
   for (int i = lane; i < 2 * TB * 3 * DMAX; i += WAVE) (&buf_[0][0][0])[i] = 0.f;   // pad rows stay zero
   __syncthreads();
   float pre[TB][PER], vpre[TB], bpre[TB];
