@@ -112,6 +112,191 @@ class GluSpec(BaseModel):
     alpha: float = 1.702
 
 
+class MaskedAttnSpec(BaseModel):
+    """GQA softmax attention without rotation whose causal mask is a sliding
+    window of ``mask_size`` positions (0 = plain causal) that also keeps the
+    first ``keep_first`` positions of the sequence; q and k pass an RMS norm
+    per head (one weight of size ``dim`` shared by the heads). ``sink``: the
+    softmax denominator holds one more term exp(0) that carries no value.
+    The concatenated heads are gated elementwise by sigmoid(W_g h)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    mask_size: int = 0
+    keep_first: int = 0
+    sink: bool = True
+
+
+class WkvSpec(BaseModel):
+    """Time mixing with a decay per head and key channel that depends on the
+    token: S <- diag(w_t) S + k v^T, read before the update with a bonus for
+    the current token; inputs are mixed with the previous token's."""
+
+    heads: int
+    dim: int
+    # bottleneck of the decay's low-rank projection; a checkpoint fixes it by
+    # its tensor shapes
+    decay_rank: int = 16
+
+
+class MlstmSpec(BaseModel):
+    """Matrix memory with exponential input gate, sigmoid forget gate (both
+    soft-capped at ``gate_cap``) and a running maximum as stabiliser."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+class RoutedExpertsSpec(BaseModel):
+    """Mixture of silu-GLU experts behind a softmax router. The last
+    ``identity`` router outputs are experts that return their input. The
+    choice is made on score + correction among the experts of the best
+    ``group_keep`` of ``group_count`` groups of neighbours."""
+
+    kind: Literal["moe"] = "moe"
+    experts: int
+    identity: int = 0
+    top: int
+    group_count: int = 1
+    group_keep: int = 1
+    ff: int
+
+
+class BigramSpec(BaseModel):
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+
+class LoopSpec(BaseModel):
+    start: int
+    stop: int
+    times: int
+
+
+class MedilixLayerSpec(BaseModel):
+    type: Literal["attention", "wkv", "mlstm"]
+    attention: Optional[MaskedAttnSpec] = None
+    wkv: Optional[WkvSpec] = None
+    mlstm: Optional[MlstmSpec] = None
+    mlp: Optional[Union[GluSpec, RoutedExpertsSpec]] = None
+
+
+class MedilixArchConfig(BaseModel):
+    """A decoder with parallel layers x <- x + mixer(norm1 x) + ff(norm2 x),
+    three mixer types (windowed attention with a sink, wkv, mlstm), dense or
+    routed feed-forwards, a grouped RMS norm, a hashed bigram embedding added
+    to the token embedding and an optional run of layers that repeats with
+    shared weights. Every size comes from the checkpoint's config.json."""
+
+    arch: Literal["medilix"] = "medilix"
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float = 1e-5
+    norm_groups: int = 1
+    embed_scale: float = 1.0
+    bigram: Optional[BigramSpec] = None
+    layers: List[MedilixLayerSpec]
+    loop: Optional[LoopSpec] = None
+    max_position_embeddings: int = 1 << 24
+    tie_word_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def layer_runs(self) -> List[tuple]:
+        """(layer index, starts a pass of the loop) per layer run, in
+        execution order: the looped range runs ``times`` times in a row."""
+        n = len(self.layers)
+        if self.loop is None:
+            return [(i, False) for i in range(n)]
+        a, b, times = self.loop.start, self.loop.stop, self.loop.times
+        looped = [(i, i == a) for i in range(a, b)] * times
+        return [(i, False) for i in range(a)] + looped + [(i, False) for i in range(b, n)]
+
+    @classmethod
+    def from_checkpoint_config(cls, d: dict, shapes: Optional[dict] = None) -> "MedilixArchConfig":
+        """Parse the family's config.json (keys: vocab, width, norm.eps,
+        norm.groups, embedding.scale / .bigram, loop, layers[].type / .mixer /
+        .mlp). ``shapes`` (tensor name -> shape, from the safetensors header)
+        supplies what config.json leaves to the tensors: the decay rank."""
+        shapes = shapes or {}
+        layers = []
+        for li, spec in enumerate(d["layers"]):
+            m = spec["mixer"]
+            mlp = spec.get("mlp")
+            ff = None
+            if mlp:
+                if mlp.get("kind", "dense") == "dense":
+                    ff = GluSpec(ff=mlp["ff"], limit=mlp["limit"])
+                elif mlp["kind"] == "moe":
+                    r = mlp["router"]
+                    grp = r.get("groups") or {}
+                    ff = RoutedExpertsSpec(experts=r["experts"], identity=r.get("identity", 0), top=r["top"],
+                                           group_count=grp.get("count", 1), group_keep=grp.get("keep", 1),
+                                           ff=mlp["expert"]["ff"])
+                else:
+                    raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+            kind = spec["type"]
+            if kind == "attention":
+                mask = m.get("mask") or {}
+                layers.append(MedilixLayerSpec(type=kind, mlp=ff, attention=MaskedAttnSpec(
+                    heads=m["heads"], kv_heads=m["kv_heads"], dim=m["dim"], vdim=m["vdim"], scale=m["scale"],
+                    mask_size=mask.get("size", 0), keep_first=mask.get("keep_first", 0))))
+            elif kind == "wkv":
+                layers.append(MedilixLayerSpec(type=kind, mlp=ff, wkv=WkvSpec(
+                    heads=m["heads"], dim=m["dim"],
+                    decay_rank=(shapes.get(f"l{li}.mix.w1") or [16])[0])))
+            elif kind == "mlstm":
+                layers.append(MedilixLayerSpec(type=kind, mlp=ff, mlstm=MlstmSpec(
+                    heads=m["heads"], dim=m["dim"], vdim=m["vdim"], gate_cap=m["gate_cap"])))
+            else:
+                raise ValueError(f"unknown layer type {kind!r}")
+        emb = d.get("embedding") or {}
+        bg = emb.get("bigram")
+        lp = d.get("loop")
+        if lp and (lp["times"] < 1 or not 0 <= lp["start"] < lp["stop"] <= len(layers)):
+            raise ValueError(f"loop {lp} does not fit {len(layers)} layers")
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], rms_norm_eps=d["norm"]["eps"],
+                   norm_groups=d["norm"].get("groups", 1), embed_scale=emb.get("scale", 1.0),
+                   bigram=BigramSpec(**bg) if bg else None, layers=layers,
+                   loop=LoopSpec(**lp) if lp else None)
+
+
+def _medilix_preset(vocab, width, depth, heads, kv_heads, dim, mask, keep, r_heads, r_dim, m_heads, m_dim,
+                    m_vdim, ff, experts, top, expert_ff, pattern="awm", loop=None, groups=2,
+                    identity=2) -> MedilixArchConfig:
+    """Random-init presets of the family: ``pattern`` repeats over the depth
+    ('a' attention + dense ff, 'w' wkv + routed experts, 'm' mlstm + dense ff)."""
+    import math as _math
+
+    layers = []
+    for i in range(depth):
+        c = pattern[i % len(pattern)]
+        dense = GluSpec(ff=ff, limit=7.0)
+        moe = RoutedExpertsSpec(experts=experts, identity=identity, top=top, group_count=2, group_keep=1,
+                                ff=expert_ff)
+        if c == "a":
+            layers.append(MedilixLayerSpec(type="attention", mlp=dense, attention=MaskedAttnSpec(
+                heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=1.0 / _math.sqrt(dim),
+                mask_size=mask, keep_first=keep)))
+        elif c == "w":
+            layers.append(MedilixLayerSpec(type="wkv", mlp=moe, wkv=WkvSpec(
+                heads=r_heads, dim=r_dim, decay_rank=max(8, width // 64))))
+        else:
+            layers.append(MedilixLayerSpec(type="mlstm", mlp=dense, mlstm=MlstmSpec(
+                heads=m_heads, dim=m_dim, vdim=m_vdim, gate_cap=15.0)))
+    return MedilixArchConfig(vocab_size=vocab, hidden_size=width, norm_groups=groups, embed_scale=1.0,
+                             bigram=BigramSpec(buckets=max(7, vocab // 2 - 1), mul_prev=131, mul_cur=5),
+                             layers=layers, loop=LoopSpec(**loop) if loop else None)
+
+
 class HybridLayerSpec(BaseModel):
     type: Literal["parallel", "channel_delta"]
     parallel: Optional[ParallelMixerSpec] = None
@@ -291,6 +476,22 @@ MODEL_PRESETS: dict = {
     "llama-1b-l6": ModelArchConfig(
         arch="llama", vocab_size=32000, hidden_size=2048, intermediate_size=8192,
         num_layers=6, num_heads=16, num_kv_heads=4, rope_theta=500000.0),
+    # Medilix family (parallel layers; windowed attention with a sink, wkv and
+    # mlstm mixers; dense and routed feed-forwards; looped layer range)
+    "tiny-medilix": _medilix_preset(
+        vocab=512, width=64, depth=4, heads=4, kv_heads=2, dim=16, mask=24, keep=3, r_heads=2, r_dim=16,
+        m_heads=2, m_dim=8, m_vdim=16, ff=96, experts=4, top=2, expert_ff=48,
+        loop={"start": 1, "stop": 3, "times": 2}),
+    "mid-medilix": _medilix_preset(
+        vocab=2048, width=512, depth=3, heads=4, kv_heads=2, dim=128, mask=256, keep=4, r_heads=8, r_dim=64,
+        m_heads=4, m_dim=64, m_vdim=128, ff=1024, experts=8, top=2, expert_ff=256),
+    # layer shapes of real models at reduced depth, beside llama-{1b,8b}-l6
+    "medilix-8b-l6": _medilix_preset(
+        vocab=32000, width=4096, depth=6, heads=32, kv_heads=8, dim=128, mask=2048, keep=4, r_heads=64,
+        r_dim=64, m_heads=32, m_dim=64, m_vdim=128, ff=14336, experts=8, top=2, expert_ff=7168, identity=0),
+    "medilix-1b-l6": _medilix_preset(
+        vocab=32000, width=2048, depth=6, heads=16, kv_heads=4, dim=128, mask=1024, keep=4, r_heads=32,
+        r_dim=64, m_heads=16, m_dim=64, m_vdim=128, ff=8192, experts=8, top=2, expert_ff=4096, identity=0),
 }
 
 
@@ -392,11 +593,12 @@ class EngineConfig(BaseModel):
             )
         with open(cfg_path) as f:
             hf = json.load(f)
-        if str(hf.get("architecture", "")).lower() == "zutalix":
+        family = str(hf.get("architecture", "")).lower()
+        if family in ("zutalix", "medilix"):
             from .weights import safetensors_shapes
 
-            return HybridArchConfig.from_checkpoint_config(
-                hf, safetensors_shapes(os.path.dirname(cfg_path)))
+            reader = HybridArchConfig if family == "zutalix" else MedilixArchConfig
+            return reader.from_checkpoint_config(hf, safetensors_shapes(os.path.dirname(cfg_path)))
         arch = "mixtral" if "mixtral" in hf.get("model_type", "").lower() or hf.get("num_local_experts") else "llama"
         return ModelArchConfig(
             arch=arch,

@@ -210,22 +210,33 @@ class LayerCacheSpec:
     """What one layer keeps between steps. kv = (kv_heads, key_dim, value_dim)
     of a paged attention cache; rec = (heads, key_dim, value_dim) of an fp32
     recurrent state matrix per head; conv = (channels, history) of carried
-    convolution inputs. None = the layer has no such state."""
+    convolution inputs; shift = width of the previous token's layer input
+    (token-shift mixers); tok = the previous token id (hashed n-gram
+    embeddings). None / False = the layer has no such state."""
 
     kv: Optional[Tuple[int, int, int]] = None
     rec: Optional[Tuple[int, int, int]] = None
     conv: Optional[Tuple[int, int]] = None
+    shift: Optional[int] = None
+    tok: bool = False
 
 
 @dataclass
 class LayerState:
     """One layer's device tensors: paged k/v [NB, G, BS, D|Dv], recurrent
-    state [slots, H, D, V] fp32, convolution history [slots, K-1, C]."""
+    state [slots, H, D, V] fp32, convolution history [slots, K-1, C], previous
+    layer input [slots, W], previous token id [slots] int32."""
 
     k: Optional[torch.Tensor] = None
     v: Optional[torch.Tensor] = None
     rec: Optional[torch.Tensor] = None
     conv: Optional[torch.Tensor] = None
+    shift: Optional[torch.Tensor] = None
+    tok: Optional[torch.Tensor] = None
+
+    def slot_tensors(self):
+        """The per-slot tensors (first dim = slot), for copying a slot."""
+        return [t for t in (self.rec, self.conv, self.shift, self.tok) if t is not None]
 
 
 class StateSlotPool:
@@ -254,7 +265,9 @@ class StateSlotPool:
 class HybridStateCache(PagedKVCache):
     """Cache and state manager for models whose layers are listed one by one
     and may each keep a paged attention cache, a recurrent state, a
-    convolution history, or several of these. Block ids are shared by all
+    convolution history, the previous token's input, or several of these. A
+    model may list more entries than it has layers (a layer that runs several
+    times keeps one entry per run; an embedding with state keeps one too). Block ids are shared by all
     attention layers (one block table per sequence), slots by all recurrent
     layers; per-layer tensors may differ in head count and sizes.
 
@@ -283,6 +296,10 @@ class HybridStateCache(PagedKVCache):
             if sp.conv is not None:
                 c, hist = sp.conv
                 st.conv = torch.zeros(num_slots, hist, c, device=device, dtype=dtype)
+            if sp.shift is not None:
+                st.shift = torch.zeros(num_slots, sp.shift, device=device, dtype=dtype)
+            if sp.tok:
+                st.tok = torch.zeros(num_slots, device=device, dtype=torch.int32)
             self.layers.append(st)
         self.allocator = BlockAllocator(num_blocks)
         self.slots = StateSlotPool(num_slots)
@@ -299,6 +316,10 @@ class HybridStateCache(PagedKVCache):
                 n += sp.rec[0] * sp.rec[1] * sp.rec[2] * 4
             if sp.conv:
                 n += sp.conv[0] * sp.conv[1] * elem
+            if sp.shift:
+                n += sp.shift * elem
+            if sp.tok:
+                n += 4
         return n
 
     def layer_caches(self) -> List[LayerState]:
@@ -336,10 +357,8 @@ class HybridStateCache(PagedKVCache):
         child.state_slot = slot
         if parent.state_slot >= 0:
             for st in self.layers:
-                if st.rec is not None:
-                    st.rec[slot].copy_(st.rec[parent.state_slot])
-                if st.conv is not None:
-                    st.conv[slot].copy_(st.conv[parent.state_slot])
+                for t in st.slot_tensors():
+                    t[slot].copy_(t[parent.state_slot])
         return child
 
     def free_sequence(self, seq: SequenceKV) -> None:

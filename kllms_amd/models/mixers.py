@@ -1,7 +1,8 @@
 """Sequence mixers and feed-forward blocks with their constants as
 parameters: block-local softmax attention over the paged cache, decayed
 linear attention, the gated delta rule with per-channel decay and short
-convolutions, and the clamped GLU. Each runs on "segment" batches
+convolutions, the clamped GLU; windowed attention with kept first tokens and
+a sink, the wkv and mlstm recurrences, and routed experts. Each runs on "segment" batches
 (ForwardBatch.seg_start / state_slots / token_seg): any mix of prompt
 portions and single decoded tokens, attention keys found through the block
 table and recurrent state carried in per-sequence slots.
@@ -22,8 +23,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from ..engine.config import (BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec,
-                             ParallelMixerSpec, RotarySpec)
+from ..engine.config import (BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec, MaskedAttnSpec,
+                             MlstmSpec, ParallelMixerSpec, RotarySpec, RoutedExpertsSpec, WkvSpec)
 from ..engine.kvcache import LayerCacheSpec, LayerState
 
 
@@ -337,3 +338,209 @@ class ClampedGLU(nn.Module):
 
     def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
         return {pre + "gate": self.inp.slot("gate"), pre + "up": self.inp.slot("up"), pre + "down": self.down}
+
+
+class WindowSinkAttention(nn.Module):
+    """GQA softmax attention over the paged cache with a sliding window that
+    also keeps the first tokens, a sink term in the denominator, an RMS norm on
+    every q and k head, no rotation, and an elementwise sigmoid gate on the
+    concatenated heads. q, k, v and the gate share one input GEMM."""
+
+    def __init__(self, spec: MaskedAttnSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert spec.heads % spec.kv_heads == 0
+        self.spec = spec
+        self.eps = eps
+        self.inp = FusedInput(hidden, [("q", spec.heads * spec.dim), ("k", spec.kv_heads * spec.dim),
+                                       ("v", spec.kv_heads * spec.vdim), ("g", spec.heads * spec.vdim)], dtype)
+        self.q_norm = _param(spec.dim, dtype=torch.float32)
+        self.k_norm = _param(spec.dim, dtype=torch.float32)
+        self.o_proj = _param(hidden, spec.heads * spec.vdim, dtype=dtype)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(kv=(sp.kv_heads, sp.dim, sp.vdim))
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        T = h.shape[0]
+        y = self.inp(h)
+        s = self.inp.split
+        q = s(y, "q").unflatten(1, (sp.heads, sp.dim))
+        k = s(y, "k").unflatten(1, (sp.kv_heads, sp.dim))
+        v = s(y, "v").unflatten(1, (sp.kv_heads, sp.vdim))
+        ops.qk_norm_store(q, k, v, self.q_norm, self.k_norm, self.eps, st.k, st.v, batch.slot_mapping)
+        att = ops.attn_window_sink(q, st, batch, sp, s(y, "g"))
+        return F.linear(att.reshape(T, -1), self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        m[pre + "q.norm"] = self.q_norm
+        m[pre + "k.norm"] = self.k_norm
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class WkvMixer(nn.Module):
+    """Time mixing with token shift. With h' the previous token's input, each
+    of r, k, v, g, w reads h + (h' - h) mu_s; r, k, v are projections of their
+    mixes, the gate is silu of its projection, the decay
+        w = exp(-exp(W_2 tanh(W_1 mix_w) + w0))
+    is per head and key channel and kept in fp32 from the mix on. Per head
+        o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T
+    then every head's o is RMS-normed, scaled by the norm weight and the gate,
+    and projected. State: S [H, D, D] fp32 and the previous input."""
+
+    STREAMS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, spec: WkvSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        self.hidden = hidden
+        hd = spec.heads * spec.dim
+        self.mu = _param(len(self.STREAMS), hidden, dtype=torch.float32)
+        self.rkvg = _param(4, hd, hidden, dtype=dtype)            # one batched GEMM for r, k, v, g
+        self.w1 = _param(spec.decay_rank, hidden, dtype=torch.float32)
+        self.w2 = _param(hd, spec.decay_rank, dtype=torch.float32)
+        self.w0 = _param(hd, dtype=torch.float32)
+        self.u = _param(spec.heads, spec.dim, dtype=torch.float32)
+        self.norm = _param(hd, dtype=torch.float32)
+        self.o_proj = _param(hidden, hd, dtype=dtype)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(rec=(sp.heads, sp.dim, sp.dim), shift=self.hidden)
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        mixes, mix_w = ops.token_shift_mix(h, self.mu, st.shift, batch.state_slots, batch.cu_seqlens,
+                                           batch.seg_start, batch.token_seg, 4)
+        y = torch.bmm(mixes, self.rkvg.transpose(1, 2))                       # [4, T, H*D]
+        d = F.linear(torch.tanh(F.linear(mix_w[0], self.w1)), self.w2)       # fp32 [T, H*D]
+        hd = (sp.heads, sp.dim)
+        o = ops.wkv_recurrence(y[0].unflatten(1, hd), y[1].unflatten(1, hd), y[2].unflatten(1, hd), d,
+                               self.w0, self.u, st.rec, batch.state_slots, batch.cu_seqlens, batch.seg_start)
+        r = ops.head_rmsnorm_gate(o, self.norm, y[3], self.eps, "silu", self.o_proj.dtype)
+        return F.linear(r, self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + "mu." + n: self.mu[i] for i, n in enumerate(self.STREAMS)}
+        for i, n in enumerate(self.STREAMS[:4]):
+            m[pre + n] = self.rkvg[i]
+        for n in ("w1", "w2", "w0", "u", "norm"):
+            m[pre + n] = getattr(self, n)
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class MlstmMixer(nn.Module):
+    """Matrix memory with a stabilised exponential input gate. Per head, with
+    i = cap tanh(z_i / cap), f = logsigmoid(cap tanh(z_f / cap)) and a running
+    maximum m (from 0):
+        m' = max(f + m, i);  S <- e^(f+m-m') S + e^(i-m') k v^T;  n likewise with k
+        o = S^T q / (max(|n . q|, e^-m') + 1e-6),  q scaled by D^-1/2
+    then RMS norm per head, norm weight, sigmoid gate, projection. The gate
+    pre-activations come from an fp32 GEMM of their own. State per head:
+    [D+1, V+1] fp32 — S, n as one more column, m in the extra row."""
+
+    def __init__(self, spec: MlstmSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        self.spec = spec
+        self.eps = eps
+        hv = spec.heads * spec.vdim
+        self.inp = FusedInput(hidden, [("q", spec.heads * spec.dim), ("k", spec.heads * spec.dim),
+                                       ("v", hv), ("g", hv)], dtype)
+        self.gates = _param(2 * spec.heads, hidden, dtype=torch.float32)    # input rows, then forget rows
+        self.gate_bias = _param(2 * spec.heads, dtype=torch.float32)
+        self.norm = _param(hv, dtype=torch.float32)
+        self.o_proj = _param(hidden, hv, dtype=dtype)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(rec=(sp.heads, sp.dim + 1, sp.vdim + 1))
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        y = self.inp(h)
+        s = self.inp.split
+        z = F.linear(h.float(), self.gates)
+        o = ops.mlstm_recurrence(s(y, "q").unflatten(1, (sp.heads, sp.dim)),
+                                 s(y, "k").unflatten(1, (sp.heads, sp.dim)),
+                                 s(y, "v").unflatten(1, (sp.heads, sp.vdim)), z, self.gate_bias, sp.gate_cap,
+                                 st.rec, batch.state_slots, batch.cu_seqlens, batch.seg_start)
+        r = ops.head_rmsnorm_gate(o, self.norm, s(y, "g"), self.eps, "sigmoid", self.o_proj.dtype)
+        return F.linear(r, self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        H = self.spec.heads
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        m[pre + "i"], m[pre + "f"] = self.gates[:H], self.gates[H:]
+        m[pre + "i.b"], m[pre + "f.b"] = self.gate_bias[:H], self.gate_bias[H:]
+        m[pre + "norm"] = self.norm
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class RoutedExperts(nn.Module):
+    """Mixture of silu-GLU experts. The router runs in fp32: scores are the
+    softmax over all outputs; the choice is made on score + correction within
+    the best groups of neighbouring experts; the chosen scores, renormalised,
+    weigh the outputs. The last ``identity`` router outputs stand for experts
+    that return their input and have no weights.
+
+    Few rows: every expert runs on every row as two batched GEMMs (the weights
+    stream from memory once either way, and shapes do not depend on the
+    routing). Many rows: rows are sorted by expert and each expert runs on its
+    slice. Both end in one weighted gather that sums a row's choices in a
+    fixed order, so a row's result does not depend on the batch around it."""
+
+    def __init__(self, spec: RoutedExpertsSpec, hidden: int, dtype):
+        super().__init__()
+        self.spec = spec
+        n = spec.experts + spec.identity
+        assert n % spec.group_count == 0 and 1 <= spec.group_keep <= spec.group_count
+        assert spec.top <= n // spec.group_count * spec.group_keep
+        self.router = _param(n, hidden, dtype=torch.float32)
+        self.correction = _param(n, dtype=torch.float32)
+        self.w_gate_up = _param(spec.experts, 2 * spec.ff, hidden, dtype=dtype)
+        self.w_down = _param(spec.experts, hidden, spec.ff, dtype=dtype)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        sp = self.spec
+        T, W = h.shape
+        E, top = sp.experts, sp.top
+        z = F.linear(h.float(), self.router)
+        idx, w = ops.moe_route(z, self.correction, top, sp.group_count, sp.group_keep)
+        if T <= 8 * E:
+            gu = torch.bmm(h.unsqueeze(0).expand(E, T, W), self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)
+            act = ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]).view(E, T, sp.ff)
+            rows = torch.bmm(act, self.w_down.transpose(1, 2)).view(E * T, W)
+            t_idx = torch.arange(T, dtype=torch.int32, device=h.device).unsqueeze(1)
+            rowidx = torch.where(idx < E, idx * T + t_idx, torch.full_like(idx, -1))
+            return ops.moe_combine(rows, h, rowidx, w, h.dtype)
+        flat = idx.reshape(-1).long().clamp(max=E)                # identity experts sort last
+        order = torch.argsort(flat, stable=True)
+        counts = torch.bincount(flat, minlength=E + 1)[:E].tolist()   # one host sync per call
+        n_real = sum(counts)
+        xs = h[(order[:n_real] // top)]
+        rows = torch.empty((max(n_real, 1), W), dtype=h.dtype, device=h.device)
+        s0 = 0
+        for e, c in enumerate(counts):
+            if c:
+                gu = F.linear(xs[s0:s0 + c], self.w_gate_up[e])
+                rows[s0:s0 + c] = F.linear(ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]), self.w_down[e])
+                s0 += c
+        pos = torch.empty(T * top, dtype=torch.int32, device=h.device)
+        pos[order] = torch.arange(T * top, dtype=torch.int32, device=h.device)
+        rowidx = torch.where(idx < E, pos.view(T, top), torch.full_like(idx, -1))
+        return ops.moe_combine(rows, h, rowidx, w, h.dtype)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        ff = self.spec.ff
+        m = {pre + "router": self.router, pre + "correction": self.correction}
+        for e in range(self.spec.experts):
+            m[f"{pre}e{e}.gate"] = self.w_gate_up[e, :ff]
+            m[f"{pre}e{e}.up"] = self.w_gate_up[e, ff:]
+            m[f"{pre}e{e}.down"] = self.w_down[e]
+        return m

@@ -18,7 +18,11 @@ def model_class(arch: str):
         from .zutalix import ZutalixForCausalLM
 
         return ZutalixForCausalLM
+    if arch == "medilix":
+        from .medilix import MedilixForCausalLM
+
+        return MedilixForCausalLM
     raise ValueError(f"no model registered for architecture {arch!r}")
 
 
-ARCHITECTURES = ("llama", "mixtral", "zutalix")
+ARCHITECTURES = ("llama", "mixtral", "zutalix", "medilix")

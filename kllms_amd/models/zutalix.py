@@ -27,6 +27,7 @@ from .. import ops
 from ..engine.config import HybridArchConfig, HybridLayerSpec
 from ..engine.kvcache import LayerCacheSpec, LayerState
 from ..parallel.tp import ParallelContext
+from .listed import ListedLayerLM
 from .llama import ForwardBatch
 from .mixers import ChannelDeltaMixer, ClampedGLU, ParallelMixer, _param
 
@@ -75,11 +76,7 @@ class HybridLayer(nn.Module):
         return m
 
 
-class ZutalixForCausalLM(nn.Module):
-    # the engine keeps a recurrent-state slot per sequence and feeds segment
-    # batches; prefix-block reuse is off (state cannot be rebuilt from blocks)
-    stateful = True
-
+class ZutalixForCausalLM(ListedLayerLM):
     def __init__(self, cfg: HybridArchConfig, ctx: Optional[ParallelContext] = None, dtype=torch.bfloat16):
         super().__init__()
         self.cfg = cfg
@@ -110,21 +107,7 @@ class ZutalixForCausalLM(nn.Module):
             m.update(layer.checkpoint_map(f"l{i}."))
         return m
 
-    @torch.no_grad()
-    def load_named_tensors_(self, named: Iterable[Tuple[str, torch.Tensor]]) -> None:
-        m = self.checkpoint_map()
-        seen = set()
-        for name, t in named:
-            dst = m.get(name)
-            if dst is None:
-                raise RuntimeError(f"checkpoint tensor {name!r} has no place in this model")
-            if tuple(dst.shape) != tuple(t.shape):
-                raise RuntimeError(f"{name}: checkpoint shape {tuple(t.shape)} != model {tuple(dst.shape)}")
-            dst.copy_(t.to(dst.dtype))
-            seen.add(name)
-        missing = sorted(set(m) - seen)
-        if missing:
-            raise RuntimeError(f"checkpoint left {len(missing)} tensors unassigned: {missing[:6]}")
+    def _after_load(self) -> None:
         self._zero_unbiased()
 
     def _zero_unbiased(self) -> None:
@@ -168,21 +151,3 @@ class ZutalixForCausalLM(nn.Module):
             if self.trace_layers is not None:
                 self.trace_layers.append(x.clone())
         return h
-
-    trace_layers: Optional[list] = None   # debugging: residual after each layer
-
-    def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        return self.lm_head(hidden).float()
-
-    def forward_prefill(self, input_ids: torch.Tensor, batch: ForwardBatch) -> torch.Tensor:
-        """Logits of the LAST row of each segment: [n_seg, V]."""
-        hidden = self.forward_hidden(input_ids, batch)
-        last_idx = (batch.cu_seqlens[1:] - 1).long()
-        return self.compute_logits(hidden[last_idx])
-
-    def forward_decode(self, input_ids: torch.Tensor, batch: ForwardBatch) -> torch.Tensor:
-        return self.compute_logits(self.forward_hidden(input_ids, batch))
-
-    def to_device(self, device) -> "ZutalixForCausalLM":
-        self.to(device)
-        return self

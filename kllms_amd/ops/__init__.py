@@ -286,17 +286,32 @@ def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mappin
     torch_ref.rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping)
 
 
-def attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_size,
-                          gate=None, row_map=None, out=None):
-    """row_map / out (GPU only): serve just the listed rows, writing into an
-    existing [T, H, Dv] tensor whose other rows another kernel fills."""
+def attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_kind, mask_size,
+                      keep_first=0, sink=False, gate=None, row_map=None, out=None):
+    """Paged softmax attention with a block-local (mask_kind 0) or sliding
+    window + kept first tokens (mask_kind 1) causal mask, optional sink term,
+    gate per head [T, H] or per element [T, H*Dv]. row_map / out (GPU only):
+    serve just the listed rows, writing into an existing [T, H, Dv] tensor
+    whose other rows another kernel fills."""
     if _gpu(q):
         if out is None:
             out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
-        _seq().attn_blocklocal_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions,
-                                     gate if gate is not None else _none(q), scale, mask_size,
-                                     row_map if row_map is not None else _none(q, torch.int32))
+        _seq().attn_masked_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions,
+                                 gate if gate is not None else _none(q), scale, int(mask_kind), int(mask_size),
+                                 int(keep_first), bool(sink),
+                                 row_map if row_map is not None else _none(q, torch.int32))
         return out
+    assert row_map is None and out is None
+    return torch_ref.attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale,
+                                       mask_kind, mask_size, keep_first, sink, gate)
+
+
+def attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_size,
+                          gate=None, row_map=None, out=None):
+    """Block-local mask, no sink, per-head gate: a case of attn_masked_paged."""
+    if _gpu(q):
+        return attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, 0, mask_size,
+                                 0, False, gate, row_map, out)
     assert row_map is None and out is None
     return torch_ref.attn_blocklocal_paged(q, k_cache, v_cache, block_tables, token_seg, positions,
                                            scale, mask_size, gate)
@@ -367,9 +382,129 @@ def gated_delta_rule(q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots,
                                       cu_seqlens, seg_start)
 
 
-def clamped_glu(gate, up, limit: float, alpha: float):
+def gated_act(gate, up, limit: float, alpha: float, up_bias: float):
+    """min(g, limit) sigmoid(alpha min(g, limit)) (clamp(u, +-limit) + up_bias)."""
     if _gpu(gate):
         out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
-        _seq().clamped_glu(out, gate, up, limit, alpha)
+        _seq().gated_act(out, gate, up, limit, alpha, up_bias)
         return out
+    return torch_ref.gated_act(gate, up, limit, alpha, up_bias)
+
+
+def clamped_glu(gate, up, limit: float, alpha: float):
+    if _gpu(gate):
+        return gated_act(gate, up, limit, alpha, 1.0)
     return torch_ref.clamped_glu(gate, up, limit, alpha)
+
+
+def silu_glu(gate, up):
+    """silu(gate) * up in the activation dtype (bf16 or fp32)."""
+    return gated_act(gate, up, float("inf"), 1.0, 0.0)
+
+
+def embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state, state_slots, cu_seqlens,
+                 seg_start, token_seg):
+    if _gpu(table):
+        out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
+        has = bigram is not None
+        _seq().embed_bigram(out, ids, table, bigram if has else _none(table), float(scale), int(mul_prev),
+                            int(mul_cur), int(buckets), tok_state if has else _none(table, torch.int32),
+                            state_slots, cu_seqlens, seg_start, token_seg)
+        return out
+    return torch_ref.embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state,
+                                  state_slots, cu_seqlens, seg_start)
+
+
+def group_norm_pair(x, a, b, w1, w2, groups, eps, out_dtype):
+    """x (fp32 residual, in place) += a + b; returns the grouped RMS norm of x
+    under two weights (the second may be None)."""
+    if _gpu(x):
+        h1 = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        h2 = torch.empty(x.shape, dtype=out_dtype, device=x.device) if w2 is not None else None
+        f = _none(x, torch.float32)
+        e = _none(x, out_dtype)
+        _seq().group_norm_pair(x, a if a is not None else e, b if b is not None else e, w1,
+                               w2 if w2 is not None else f, h1, h2 if h2 is not None else e, int(groups), eps)
+        return h1, h2
+    return torch_ref.group_norm_pair(x, a, b, w1, w2, groups, eps, out_dtype)
+
+
+def cast_concat(x, x0, a, b, out_dtype):
+    """x (fp32 residual, in place) += a + b; returns [x | x0] in out_dtype."""
+    if _gpu(x):
+        out = torch.empty((x.shape[0], 2 * x.shape[1]), dtype=out_dtype, device=x.device)
+        e = _none(x, out_dtype)
+        _seq().cast_concat(out, x, x0, a if a is not None else e, b if b is not None else e)
+        return out
+    return torch_ref.cast_concat(x, x0, a, b, out_dtype)
+
+
+def qk_norm_store(q, k, v, wq, wk, eps, k_cache, v_cache, slot_mapping) -> None:
+    if _gpu(q):
+        _seq().qk_norm_store(q, k, v, wq, wk, eps, k_cache, v_cache, slot_mapping)
+        return
+    torch_ref.qk_norm_store(q, k, v, wq, wk, eps, k_cache, v_cache, slot_mapping)
+
+
+def token_shift_mix(h, mu, shift_state, state_slots, cu_seqlens, seg_start, token_seg, n_act):
+    """([n_act, T, W] in h's dtype, [n - n_act, T, W] fp32) mixes of each row
+    with its predecessor; carries the last row in shift_state."""
+    if _gpu(h):
+        T, W = h.shape
+        n = mu.shape[0]
+        act = torch.empty((n_act, T, W), dtype=h.dtype, device=h.device)
+        f32 = torch.empty((n - n_act, T, W), dtype=torch.float32, device=h.device)
+        _seq().token_shift_mix(act, f32, h, mu, shift_state, state_slots, cu_seqlens, seg_start, token_seg)
+        return act, f32
+    return torch_ref.token_shift_mix(h, mu, shift_state, state_slots, cu_seqlens, seg_start, n_act, h.dtype)
+
+
+def wkv_recurrence(r, k, v, d, w0, u, state, state_slots, cu_seqlens, seg_start):
+    if _gpu(r):
+        o = torch.empty((r.shape[0], r.shape[1], v.shape[2]), dtype=torch.float32, device=r.device)
+        _seq().wkv_recurrence(o, r, k, v, d, w0, u, state, state_slots, cu_seqlens, seg_start)
+        return o
+    return torch_ref.wkv_recurrence(r, k, v, d, w0, u, state, state_slots, cu_seqlens, seg_start)
+
+
+def mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens, seg_start):
+    if _gpu(q):
+        o = torch.empty((q.shape[0], q.shape[1], v.shape[2]), dtype=torch.float32, device=q.device)
+        _seq().mlstm_recurrence(o, q, k, v, gates, gate_bias, float(cap), state, state_slots, cu_seqlens,
+                                seg_start)
+        return o
+    return torch_ref.mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens,
+                                      seg_start)
+
+
+def head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype):
+    if _gpu(o):
+        out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
+        _seq().head_rmsnorm_gate(out, o, weight, gate, eps, 0 if gate_act == "sigmoid" else 1)
+        return out
+    return torch_ref.head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype)
+
+
+def moe_route(z, correction, top, group_count, group_keep):
+    if _gpu(z):
+        idx = torch.empty((z.shape[0], top), dtype=torch.int32, device=z.device)
+        w = torch.empty((z.shape[0], top), dtype=torch.float32, device=z.device)
+        _seq().moe_route(idx, w, z, correction, int(top), int(group_count), int(group_keep))
+        return idx, w
+    return torch_ref.moe_route(z, correction, top, group_count, group_keep)
+
+
+def moe_combine(rows, h, rowidx, w, out_dtype):
+    if _gpu(h):
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        _seq().moe_combine(out, rows, h, rowidx, w)
+        return out
+    return torch_ref.moe_combine(rows, h, rowidx, w, out_dtype)
+
+
+def attn_window_sink(q, st, batch, spec, gate):
+    """Windowed attention with kept first tokens and a sink for one step's
+    rows, keys through the block table (prompt portions, decoded tokens and
+    mixes alike)."""
+    return attn_masked_paged(q, st.k, st.v, batch.block_tables, batch.token_seg, batch.positions, spec.scale,
+                             1, spec.mask_size, spec.keep_first, spec.sink, gate)

@@ -1,5 +1,6 @@
-// Rotary (interleaved pairs, partial width) + paged K/V store, and block-local
-// softmax attention over the paged cache. One kernel serves prompt portions,
+// Rotary (interleaved pairs, partial width) + paged K/V store, q/k head norm +
+// paged store, and masked softmax attention over the paged cache (block-local
+// or sliding-window mask with kept first tokens, optional sink term). One kernel serves prompt portions,
 // single decoded tokens and mixed batches: every query row finds its keys
 // through its segment's block table, so the result does not depend on how the
 // prompt was cut into steps.
@@ -58,11 +59,58 @@ __global__ void rope_pairs_store_kernel(T* __restrict__ q, const T* __restrict__
   }
 }
 
-// grid (T, H), one wave per (query row, head). Keys lo..p, lo = the start of
-// p's aligned block of mask_size positions (0 when mask_size == 0), in tiles of
-// 64: lane j scores key lo + tile*64 + j (q staged in LDS), the tile's weights
+// grid (T, H + G), one wave per (row, head): RMS norm over the head's D
+// entries with a weight shared by the heads. Query heads are normed in place;
+// key heads go normed into k_cache, their value rows into v_cache.
+template <typename T>
+__global__ void qk_norm_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                     const float* __restrict__ wq, const float* __restrict__ wk, float eps,
+                                     T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     const int64_t* __restrict__ slots, int H, int G, int D, int Dv, int BS,
+                                     int q_stride, int k_stride, int v_stride) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const bool is_q = h < H;
+  const int g = h - H;
+  const T* src = is_q ? q + (int64_t)t * q_stride + (int64_t)h * D : k + (int64_t)t * k_stride + (int64_t)g * D;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += WAVE) { const float x = ldf(src + i); ss += x * x; }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)D + eps);
+  if (is_q) {
+    T* dst = q + (int64_t)t * q_stride + (int64_t)h * D;
+    for (int i = lane; i < D; i += WAVE) stf(dst + i, ldf(src + i) * r * wq[i]);
+    return;
+  }
+  const int64_t slot = slots[t];
+  const int64_t blk = slot / BS, off = slot % BS;
+  T* kc = k_cache + ((blk * G + g) * BS + off) * D;
+  T* vc = v_cache + ((blk * G + g) * BS + off) * Dv;
+  for (int i = lane; i < D; i += WAVE) stf(kc + i, ldf(src + i) * r * wk[i]);
+  const T* vrow = v + (int64_t)t * v_stride + (int64_t)g * Dv;
+  for (int i = lane; i < Dv; i += WAVE) vc[i] = vrow[i];
+}
+
+// The keys that position p sees, as nk kept first positions 0..nk-1 followed by
+// lo..p. mask_kind 0: lo = the start of p's aligned block of mask_size
+// positions, nothing kept. mask_kind 1: a window of mask_size positions ending
+// at p, plus the first keep_first positions of the sequence. mask_size 0 =
+// plain causal. Visible key number u (0 <= u < nk + p - lo + 1) is position
+// u < nk ? u : lo + u - nk.
+__device__ __forceinline__ void mask_range(int mask_kind, int mask_size, int keep_first, int p, int& lo,
+                                           int& nk) {
+  lo = 0; nk = 0;
+  if (mask_size <= 0) return;
+  if (mask_kind == 0) { lo = (p / mask_size) * mask_size; return; }
+  lo = max(0, p - mask_size + 1);
+  nk = min(keep_first, lo);
+}
+
+// grid (T, H), one wave per (query row, head). The visible keys in tiles of
+// 64: lane u scores visible key tile*64 + u (q staged in LDS), the tile's weights
 // go through LDS, then lanes own output dims and sweep the tile's value rows.
-// Online softmax in fp32. Optional per-head sigmoid gate on the output.
+// Online softmax in fp32; with a sink the running (max, sum) starts at (0, 1):
+// one more key of score 0 that carries no value. Optional sigmoid gate on the
+// output: gate_kind 1 = one logit per head [T, H], 2 = per element [T, H*Dv].
 #define ATTN_MAX_ACC 8   // Dv <= 512
 template <typename T>
 __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __restrict__ q,
@@ -71,7 +119,8 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
                                              const int* __restrict__ token_seg,
                                              const int64_t* __restrict__ positions,
                                              const T* __restrict__ gate, const int* __restrict__ row_map,
-                                             float scale, int mask_size,
+                                             float scale, int mask_kind, int mask_size, int keep_first,
+                                             int sink, int gate_kind,
                                              int H, int G, int D, int Dv, int BS, int bt_stride,
                                              int q_stride, int gate_stride) {
   extern __shared__ float lds[];       // q [D] | p [64] | key row index [64] (as int)
@@ -84,7 +133,9 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
   const int h = blockIdx.y, lane = threadIdx.x;
   const int g = h / (H / G);
   const int p = (int)positions[t];
-  const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
+  int lo, nk;
+  mask_range(mask_kind, mask_size, keep_first, p, lo, nk);
+  const int total = nk + (p - lo + 1);
   const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
   const T* qrow = q + (int64_t)t * q_stride + (int64_t)h * D;
   for (int i = lane; i < D; i += WAVE) qs[i] = ldf(qrow + i) * scale;
@@ -93,12 +144,13 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
   float acc[ATTN_MAX_ACC];
 #pragma unroll
   for (int i = 0; i < ATTN_MAX_ACC; ++i) acc[i] = 0.f;
-  float m = -INFINITY, l = 0.f;
-  for (int base = lo; base <= p; base += WAVE) {
-    const int j = base + lane;
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  for (int base = 0; base < total; base += WAVE) {
+    const int u = base + lane;
     float s = -INFINITY;
     int row = -1;
-    if (j <= p) {
+    if (u < total) {
+      const int j = u < nk ? u : lo + (u - nk);
       row = (bt[j / BS] * G + g) * BS + (j % BS);
       const T* kr = k_cache + (int64_t)row * D;
       float d = 0.f;
@@ -106,14 +158,14 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
       s = d;
     }
     const float m_new = fmaxf(m, wave_max(s));
-    const float w = j <= p ? expf(s - m_new) : 0.f;
+    const float w = u < total ? expf(s - m_new) : 0.f;
     const float corr = expf(m - m_new);        // m = -inf on the first tile -> 0
     l = l * corr + wave_sum(w);
     m = m_new;
     ps[lane] = w;
     rows[lane] = row;
     __syncthreads();
-    const int n = min(WAVE, p - base + 1);
+    const int n = min(WAVE, total - base);
 #pragma unroll
     for (int i = 0; i < ATTN_MAX_ACC; ++i) acc[i] *= corr;
     for (int jj = 0; jj < n; ++jj) {
@@ -128,12 +180,13 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
     __syncthreads();
   }
   float gsc = 1.0f / l;
-  if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+  if (gate_kind == 1) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
   T* orow = out + ((int64_t)t * H + h) * Dv;
+  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)h * Dv;
 #pragma unroll
   for (int i = 0; i < ATTN_MAX_ACC; ++i) {
     const int d = lane + i * WAVE;
-    if (d < Dv) stf(orow + d, acc[i] * gsc);
+    if (d < Dv) stf(orow + d, acc[i] * gsc * (gate_kind == 2 ? sigmoid_exact(ldf(grow + d)) : 1.0f));
   }
 }
 
@@ -154,8 +207,8 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ token_seg,
     const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
-    float scale, int mask_size, int H, int G, int D, int Dv, int BS, int bt_stride, int q_stride,
-    int gate_stride) {
+    float scale, int mask_kind, int mask_size, int keep_first, int sink, int gate_kind, int H, int G, int D,
+    int Dv, int BS, int bt_stride, int q_stride, int gate_stride) {
   // The block's waves take the key tiles in turn (tile r*NW + wave in pass
   // r), each with its own running max / sum / accumulator; the partial
   // results are merged through LDS at the end. Every wave runs every pass —
@@ -171,7 +224,9 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
   int* rows = rows_[wave];
   const int g = h / (H / G);
   const int p = (int)positions[t];
-  const int lo = mask_size > 0 ? (p / mask_size) * mask_size : 0;
+  int lo, nk;
+  mask_range(mask_kind, mask_size, keep_first, p, lo, nk);
+  const int total = nk + (p - lo + 1);
   const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
   const int LPK = D / 8, KPI = WAVE / LPK, kpart = lane % LPK, kgrp = lane / LPK;
   const int LPV = Dv / 8, KPV = WAVE / LPV, vpart = lane % LPV, vgrp = lane / LPV;
@@ -180,13 +235,16 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
 #pragma unroll
   for (int e = 0; e < 8; ++e) qv[e] *= scale;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  const int ntiles = (p - lo) / WAVE + 1;
+  // the sink is one more key of score 0 without a value, held by wave 0
+  const bool sunk = sink && wave == 0;
+  float m = sunk ? 0.f : -INFINITY, l = sunk ? 1.f : 0.f;
+  const int ntiles = (total + WAVE - 1) / WAVE;
   for (int r = 0; r * NW < ntiles; ++r) {
-    const int base = lo + (r * NW + wave) * WAVE;
-    const int n = min(WAVE, p - base + 1);            // <= 0: no tile for this wave in this pass
-    const int j = base + lane;
-    rows[lane] = (n > 0 && j <= p) ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
+    const int base = (r * NW + wave) * WAVE;
+    const int n = min(WAVE, total - base);            // <= 0: no tile for this wave in this pass
+    const int u = base + lane;
+    const int j = u < nk ? u : lo + (u - nk);
+    rows[lane] = (n > 0 && u < total) ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
     __syncthreads();
     for (int it = 0; it * KPI < n; ++it) {
       const int key = it * KPI + kgrp;
@@ -251,9 +309,15 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
       for (int e = 0; e < 8; ++e) o8[e] += part_acc[w2][vpart * 8 + e] * f;
     }
     float gsc = 1.0f / L;
-    if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+    if (gate_kind == 1) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
 #pragma unroll
     for (int e = 0; e < 8; ++e) o8[e] *= gsc;
+    if (gate_kind == 2) {
+      float g8[8];
+      ld8(gate + (int64_t)t * gate_stride + (int64_t)h * Dv + vpart * 8, g8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o8[e] *= sigmoid_exact(g8[e]);
+    }
     st8(out + ((int64_t)t * H + h) * Dv + vpart * 8, o8);
   }
 }
@@ -304,28 +368,40 @@ extern "C" void seq_launch_rope_pairs_store(void* q, const void* k, const void* 
                                         v_stride);)
 }
 
-extern "C" void seq_launch_attn_blocklocal_paged(void* out, const void* q, const void* k_cache,
-                                                 const void* v_cache, const int* block_tables,
-                                                 const int* token_seg, const int64_t* positions,
-                                                 const void* gate, const int* row_map, int n_rows,
-                                                 float scale, int mask_size, int T_, int H,
-                                                 int G, int D, int Dv, int BS, int bt_stride, int q_stride,
-                                                 int gate_stride, int is_f32, hipStream_t st) {
+extern "C" void seq_launch_qk_norm_store(void* q, const void* k, const void* v, const float* wq,
+                                         const float* wk, float eps, void* k_cache, void* v_cache,
+                                         const int64_t* slots, int T_, int H, int G, int D, int Dv, int BS,
+                                         int q_stride, int k_stride, int v_stride, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(qk_norm_store_kernel<T>, dim3(T_, H + G), dim3(WAVE), 0, st, (T*)q,
+                                        (const T*)k, (const T*)v, wq, wk, eps, (T*)k_cache, (T*)v_cache, slots,
+                                        H, G, D, Dv, BS, q_stride, k_stride, v_stride);)
+}
+
+extern "C" void seq_launch_attn_masked_paged(void* out, const void* q, const void* k_cache,
+                                             const void* v_cache, const int* block_tables,
+                                             const int* token_seg, const int64_t* positions,
+                                             const void* gate, const int* row_map, int n_rows,
+                                             float scale, int mask_kind, int mask_size, int keep_first,
+                                             int sink, int gate_kind, int T_, int H,
+                                             int G, int D, int Dv, int BS, int bt_stride, int q_stride,
+                                             int gate_stride, int is_f32, hipStream_t st) {
   const size_t lds = (size_t)(D + 2 * WAVE) * sizeof(float);
   const int rows = row_map ? n_rows : T_;
   const int lpk = D / 8, lpv = Dv / 8;
   if (D % 8 == 0 && Dv % 8 == 0 && lpk <= 64 && lpv <= 64 && (lpk & (lpk - 1)) == 0 && (lpv & (lpv - 1)) == 0 &&
-      q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out)) {
+      q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out) &&
+      (gate_kind != 2 || (gate_stride % 8 == 0 && aligned16(gate)))) {
     DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE * ATTN_V8_WAVES), 0, st,
                                           (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
                                           block_tables, token_seg, positions, (const T*)gate, row_map, scale,
-                                          mask_size, H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
+                                          mask_kind, mask_size, keep_first, sink, gate_kind, H, G, D, Dv, BS,
+                                          bt_stride, q_stride, gate_stride);)
     return;
   }
   DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(rows, H), dim3(WAVE), lds, st,
                                         (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
                                         block_tables, token_seg, positions, (const T*)gate, row_map, scale,
-                                        mask_size,
+                                        mask_kind, mask_size, keep_first, sink, gate_kind,
                                         H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
 }
 

@@ -225,24 +225,25 @@ __global__ void gated_rmsnorm_rows_kernel(T* __restrict__ out, const float* __re
   st8(out + row * S + i, v);
 }
 
-// y = min(g, lim) * sigmoid(alpha * min(g, lim)) * (clamp(u, -lim, lim) + 1)
+// y = min(g, lim) * sigmoid(alpha * min(g, lim)) * (clamp(u, -lim, lim) + up_bias);
+// lim = inf, alpha = 1, up_bias = 0 is silu(g) * u
 template <typename T>
 __global__ void clamped_glu_kernel(T* __restrict__ out, const T* __restrict__ gate,
                                    const T* __restrict__ up, int64_t n, int cols, int stride,
-                                   float limit, float alpha) {
+                                   float limit, float alpha, float up_bias) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = i / cols, c = i - r * cols;
     float g = fminf(ldf(gate + r * stride + c), limit);
     float u = fminf(fmaxf(ldf(up + r * stride + c), -limit), limit);
-    stf(out + i, g * sigmoid_exact(alpha * g) * (u + 1.0f));
+    stf(out + i, g * sigmoid_exact(alpha * g) * (u + up_bias));
   }
 }
 
 template <typename T>
 __global__ void clamped_glu_v8_kernel(T* __restrict__ out, const T* __restrict__ gate,
                                       const T* __restrict__ up, int64_t n8, int cols8, int stride,
-                                      float limit, float alpha) {
+                                      float limit, float alpha, float up_bias) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = i / cols8, c = (i - r * cols8) * 8;
@@ -252,7 +253,7 @@ __global__ void clamped_glu_v8_kernel(T* __restrict__ out, const T* __restrict__
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float gc = fminf(g[e], limit), uc = fminf(fmaxf(u[e], -limit), limit);
-      g[e] = gc * sigmoid_exact(alpha * gc) * (uc + 1.0f);
+      g[e] = gc * sigmoid_exact(alpha * gc) * (uc + up_bias);
     }
     st8(out + i * 8, g);
   }
@@ -321,17 +322,18 @@ extern "C" void seq_launch_gated_rmsnorm(void* out, const float* o, const float*
                                         o, w, (const T*)gate, S, gate_stride, eps);)
 }
 
-extern "C" void seq_launch_clamped_glu(void* out, const void* gate, const void* up, int64_t rows, int cols,
-                                       int stride, float limit, float alpha, int is_f32, hipStream_t st) {
+extern "C" void seq_launch_gated_act(void* out, const void* gate, const void* up, int64_t rows, int cols,
+                                     int stride, float limit, float alpha, float up_bias, int is_f32,
+                                     hipStream_t st) {
   if (cols % 8 == 0 && stride % 8 == 0 && aligned16(out) && aligned16(gate) && aligned16(up)) {
     const int64_t n8 = rows * cols / 8;
     const int g8 = (int)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
     DISPATCH_T(is_f32, hipLaunchKernelGGL(clamped_glu_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)out,
-                                          (const T*)gate, (const T*)up, n8, cols / 8, stride, limit, alpha);)
+                                          (const T*)gate, (const T*)up, n8, cols / 8, stride, limit, alpha, up_bias);)
     return;
   }
   const int64_t n = rows * cols;
   const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(clamped_glu_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
-                                        (const T*)gate, (const T*)up, n, cols, stride, limit, alpha);)
+                                        (const T*)gate, (const T*)up, n, cols, stride, limit, alpha, up_bias);)
 }

@@ -1,0 +1,294 @@
+// Kernels of the parallel-layer family: hashed bigram embedding, the grouped
+// RMS norm fused with the residual add of two branches, the loop-entry
+// concatenation, per-head norm + gate after a recurrence, token shift, the
+// expert router and the weighted gather that combines expert outputs.
+// The residual stream, norms, router and gates are fp32; T is the activation
+// type (bf16 when serving, fp32 in exact mode).
+
+#include "seq_common.h"
+
+// ---- embedding: table[id] * scale + bigram[hash(prev, id)] -------------------
+// The previous token of a segment's first row is the sequence's carried token
+// (tok_state[slot]); a sequence's very first token takes the table's last row.
+template <typename T>
+__global__ void embed_bigram_kernel(float* __restrict__ out, const int64_t* __restrict__ ids,
+                                    const T* __restrict__ table, const T* __restrict__ bigram, float scale,
+                                    int mul_prev, int mul_cur, int buckets, const int* __restrict__ tok_state,
+                                    const int* __restrict__ slots, const int* __restrict__ cu,
+                                    const int* __restrict__ seg_start, const int* __restrict__ token_seg, int W) {
+  const int t = blockIdx.x;
+  const int64_t id = ids[t];
+  const T* erow = table + id * W;
+  const T* brow = nullptr;
+  if (bigram != nullptr) {
+    const int b = token_seg[t];
+    int64_t row;
+    if (t == cu[b] && seg_start[b] == 0) {
+      row = buckets;
+    } else {
+      const int64_t prev = t == cu[b] ? (int64_t)tok_state[slots[b]] : ids[t - 1];
+      row = (prev * mul_prev + id * mul_cur) % buckets;
+    }
+    brow = bigram + row * W;
+  }
+  float* orow = out + (int64_t)t * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    orow[i] = ldf(erow + i) * scale + (brow ? ldf(brow + i) : 0.f);
+}
+
+// after the rows are embedded: the segment's last id becomes the carried token
+__global__ void tok_state_update_kernel(const int64_t* __restrict__ ids, int* __restrict__ tok_state,
+                                        const int* __restrict__ slots, const int* __restrict__ cu, int B) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  if (cu[b + 1] > cu[b]) tok_state[slots[b]] = (int)ids[cu[b + 1] - 1];
+}
+
+// ---- residual add + grouped RMS norm under two weights ------------------------
+// x += a + b (branches optional); n = x with each of `groups` equal runs divided
+// by its own sqrt(mean square + eps); out1 = n * w1, out2 = n * w2 (optional).
+// One workgroup per row, the updated row staged in LDS between the passes.
+template <typename T>
+__global__ void group_norm_pair_kernel(float* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b,
+                                       const float* __restrict__ w1, const float* __restrict__ w2,
+                                       T* __restrict__ out1, T* __restrict__ out2, int W, int groups, float eps) {
+  extern __shared__ float row[];          // [W] | per-group 1/rms [groups]
+  __shared__ float scratch[16];
+  float* rinv = row + W;
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * W;
+  const int gs = W / groups;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = xr[i];
+    if (a != nullptr) v += ldf(a + t * W + i);
+    if (b != nullptr) v += ldf(b + t * W + i);
+    row[i] = v;
+    if (a != nullptr) xr[i] = v;
+  }
+  __syncthreads();
+  for (int g = 0; g < groups; ++g) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < gs; i += blockDim.x) { const float v = row[g * gs + i]; ss += v * v; }
+    ss = block_sum(ss, scratch);
+    if (threadIdx.x == 0) rinv[g] = 1.0f / sqrtf(ss / (float)gs + eps);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float n = row[i] * rinv[i / gs];
+    stf(out1 + t * W + i, n * w1[i]);
+    if (out2 != nullptr) stf(out2 + t * W + i, n * w2[i]);
+  }
+}
+
+// ---- loop entry: x += a + b, out = [x | x0] in the activation type ---------------
+template <typename T>
+__global__ void cast_concat_kernel(T* __restrict__ out, float* __restrict__ x, const float* __restrict__ x0,
+                                   const T* __restrict__ a, const T* __restrict__ b, int W) {
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = x[t * W + i];
+    if (a != nullptr) {
+      v += ldf(a + t * W + i);
+      if (b != nullptr) v += ldf(b + t * W + i);
+      x[t * W + i] = v;
+    }
+    stf(out + t * 2 * W + i, v);
+    stf(out + t * 2 * W + W + i, x0[t * W + i]);
+  }
+}
+
+// ---- per-head RMS norm, full-width weight, activated gate ------------------------
+// o [T, H, S] fp32; out[t, h*S + i] = o / rms(o[t,h,:]) * w[h*S + i] * act(gate[t, h*S + i]);
+// act = sigmoid (0) or silu (1). One wave per (row, head).
+template <typename T>
+__global__ void head_rmsnorm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                         const float* __restrict__ w, const T* __restrict__ gate, int H, int S,
+                                         int gate_stride, float eps, int gate_act) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const float* orow = o + (t * H + h) * S;
+  float ss = 0.f;
+  for (int i = lane; i < S; i += WAVE) { const float v = orow[i]; ss += v * v; }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)S + eps);
+  const T* grow = gate + t * gate_stride + (int64_t)h * S;
+  for (int i = lane; i < S; i += WAVE) {
+    const float g = ldf(grow + i);
+    const float ga = gate_act == 0 ? sigmoid_exact(g) : silu_exact(g);
+    stf(out + (t * H + h) * S + i, orow[i] * r * w[(int64_t)h * S + i] * ga);
+  }
+}
+
+// ---- token shift: mixes of a row with its predecessor -----------------------------
+// out[s][t] = h[t] + (prev[t] - h[t]) * mu[s]; the first n_act mixes are written in
+// the activation type, the rest in fp32. prev of a segment's first row is the
+// carried row (zeros for a fresh sequence).
+template <typename T>
+__global__ void token_shift_mix_kernel(T* __restrict__ act, float* __restrict__ f32, const T* __restrict__ h,
+                                       const float* __restrict__ mu, const T* __restrict__ shift_state,
+                                       const int* __restrict__ slots, const int* __restrict__ cu,
+                                       const int* __restrict__ seg_start, const int* __restrict__ token_seg,
+                                       int T_, int W, int n, int n_act) {
+  const int64_t t = blockIdx.x;
+  const int b = token_seg[t];
+  const bool first = t == cu[b];
+  const bool fresh = seg_start[b] == 0;
+  const T* prow = first ? shift_state + (int64_t)slots[b] * W : h + (t - 1) * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float hv = ldf(h + t * W + i);
+    const float pv = (first && fresh) ? 0.f : ldf(prow + i);
+    const float d = pv - hv;
+    for (int s = 0; s < n; ++s) {
+      const float v = hv + d * mu[(int64_t)s * W + i];
+      if (s < n_act) stf(act + ((int64_t)s * T_ + t) * W + i, v);
+      else f32[((int64_t)(s - n_act) * T_ + t) * W + i] = v;
+    }
+  }
+}
+
+template <typename T>
+__global__ void shift_state_update_kernel(const T* __restrict__ h, T* __restrict__ shift_state,
+                                          const int* __restrict__ slots, const int* __restrict__ cu, int W) {
+  const int b = blockIdx.x;
+  if (cu[b + 1] <= cu[b]) return;
+  const T* src = h + (int64_t)(cu[b + 1] - 1) * W;
+  T* dst = shift_state + (int64_t)slots[b] * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) dst[i] = src[i];
+}
+
+// ---- router --------------------------------------------------------------------
+// One wave per row. s = softmax(z) over the N outputs; c = s + correction; the
+// outputs form `gc` equal groups of neighbours, a group's score is its largest
+// c, the best `gk` groups stay eligible; the `top` eligible outputs with the
+// largest c are chosen (ties: the lower index). w = chosen s / (sum + 1e-20).
+#define ROUTE_MAX_N 256
+__global__ void __launch_bounds__(WAVE) moe_route_kernel(int* __restrict__ idx, float* __restrict__ wout,
+                                                         const float* __restrict__ z,
+                                                         const float* __restrict__ corr, int N, int top, int gc,
+                                                         int gk) {
+  __shared__ float cs[ROUTE_MAX_N], ss[ROUTE_MAX_N], gmax[ROUTE_MAX_N];
+  __shared__ int ok[ROUTE_MAX_N];
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* zr = z + t * N;
+  float mx = -INFINITY;
+  for (int e = lane; e < N; e += WAVE) mx = fmaxf(mx, zr[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < N; e += WAVE) { const float p = expf(zr[e] - mx); ss[e] = p; sum += p; }
+  sum = wave_sum(sum);
+  for (int e = lane; e < N; e += WAVE) { ss[e] /= sum; cs[e] = ss[e] + corr[e]; }
+  __syncthreads();
+  const int per = N / gc;
+  for (int g = lane; g < gc; g += WAVE) {
+    float m = -INFINITY;
+    for (int i = 0; i < per; ++i) m = fmaxf(m, cs[g * per + i]);
+    gmax[g] = m;
+    ok[g] = 0;
+  }
+  __syncthreads();
+  if (lane == 0) {
+    for (int r = 0; r < gk; ++r) {
+      int best = -1;
+      for (int g = 0; g < gc; ++g)
+        if (!ok[g] && (best < 0 || gmax[g] > gmax[best])) best = g;
+      ok[best] = 1;
+    }
+  }
+  __syncthreads();
+  float wsum = 0.f, mine = 0.f;       // lane j keeps the j-th choice's score
+  for (int r = 0; r < top; ++r) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < N; e += WAVE) {
+      if (ok[e / per] && (cs[e] > bv)) { bv = cs[e]; bi = e; }       // ascending e: ties keep the lower index
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off);
+      const int oi = __shfl_xor(bi, off);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const float sv = ss[bi];
+    wsum += sv;
+    if (lane == r) mine = sv;
+    if (lane == 0) { idx[t * top + r] = bi; cs[bi] = -INFINITY; }
+    __syncthreads();
+  }
+  if (lane < top) wout[t * top + lane] = mine / (wsum + 1e-20f);
+}
+
+// ---- combine: out[t] = sum_j w[t,j] * (rowidx[t,j] >= 0 ? rows[rowidx[t,j]] : h[t]) ------
+template <typename T>
+__global__ void moe_combine_kernel(T* __restrict__ out, const T* __restrict__ rows, const T* __restrict__ h,
+                                   const int* __restrict__ rowidx, const float* __restrict__ w, int W, int top) {
+  const int64_t t = blockIdx.x;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const int r = rowidx[t * top + j];
+      acc += w[t * top + j] * (r >= 0 ? ldf(rows + (int64_t)r * W + i) : ldf(h + t * W + i));
+    }
+    stf(out + t * W + i, acc);
+  }
+}
+
+#define DISPATCH_T(is_f32, ...)                                  \
+  if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
+
+static inline int row_threads(int W) { return W >= 1024 ? 256 : (W >= 256 ? 128 : 64); }
+
+extern "C" void seq_launch_embed_bigram(float* out, const int64_t* ids, const void* table, const void* bigram,
+                                        float scale, int mul_prev, int mul_cur, int buckets, int* tok_state,
+                                        const int* slots, const int* cu, const int* seg_start,
+                                        const int* token_seg, int T_, int B, int W, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(embed_bigram_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, out, ids,
+                                        (const T*)table, (const T*)bigram, scale, mul_prev, mul_cur, buckets,
+                                        tok_state, slots, cu, seg_start, token_seg, W);)
+  if (bigram != nullptr)
+    hipLaunchKernelGGL(tok_state_update_kernel, dim3((B + 63) / 64), dim3(64), 0, st, ids, tok_state, slots, cu, B);
+}
+
+extern "C" void seq_launch_group_norm_pair(float* x, const void* a, const void* b, const float* w1,
+                                           const float* w2, void* out1, void* out2, int T_, int W, int groups,
+                                           float eps, int is_f32, hipStream_t st) {
+  const size_t lds = (size_t)(W + groups) * sizeof(float);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(group_norm_pair_kernel<T>, dim3(T_), dim3(row_threads(W)), lds, st, x,
+                                        (const T*)a, (const T*)b, w1, w2, (T*)out1, (T*)out2, W, groups, eps);)
+}
+
+extern "C" void seq_launch_cast_concat(void* out, float* x, const float* x0, const void* a, const void* b,
+                                       int T_, int W, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(cast_concat_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)out, x,
+                                        x0, (const T*)a, (const T*)b, W);)
+}
+
+extern "C" void seq_launch_head_rmsnorm_gate(void* out, const float* o, const float* w, const void* gate,
+                                             int T_, int H, int S, int gate_stride, float eps, int gate_act,
+                                             int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(head_rmsnorm_gate_kernel<T>, dim3(T_, H), dim3(WAVE), 0, st, (T*)out, o,
+                                        w, (const T*)gate, H, S, gate_stride, eps, gate_act);)
+}
+
+extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h, const float* mu,
+                                           void* shift_state, const int* slots, const int* cu,
+                                           const int* seg_start, const int* token_seg, int T_, int B, int W,
+                                           int n, int n_act, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32,
+             hipLaunchKernelGGL(token_shift_mix_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)act, f32,
+                                (const T*)h, mu, (const T*)shift_state, slots, cu, seg_start, token_seg, T_, W, n,
+                                n_act);
+             hipLaunchKernelGGL(shift_state_update_kernel<T>, dim3(B), dim3(row_threads(W)), 0, st, (const T*)h,
+                                (T*)shift_state, slots, cu, W);)
+}
+
+extern "C" void seq_launch_moe_route(int* idx, float* w, const float* z, const float* corr, int T_, int N,
+                                     int top, int gc, int gk, hipStream_t st) {
+  hipLaunchKernelGGL(moe_route_kernel, dim3(T_), dim3(WAVE), 0, st, idx, w, z, corr, N, top, gc, gk);
+}
+
+extern "C" void seq_launch_moe_combine(void* out, const void* rows, const void* h, const int* rowidx,
+                                       const float* w, int T_, int W, int top, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)out,
+                                        (const T*)rows, (const T*)h, rowidx, w, W, top);)
+}

@@ -445,3 +445,250 @@ def clamped_glu(gate, up, limit: float, alpha: float) -> torch.Tensor:
     g = gate.float().clamp(max=limit)
     u = up.float().clamp(-limit, limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate.dtype)
+
+
+# --- parallel-layer family: grouped norm, hashed bigram embedding, windowed
+# attention with a sink, wkv and mlstm recurrences, routed experts ------------
+
+def embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state, state_slots,
+                 cu_seqlens, seg_start) -> torch.Tensor:
+    """fp32 rows table[id] * scale + bigram[(prev * mul_prev + id * mul_cur) % buckets];
+    a sequence's first token takes row ``buckets``. The previous token of a
+    segment's first row comes from tok_state [slots] (int32), which is then set
+    to the segment's last id."""
+    x = table[ids].float() * scale
+    if bigram is None:
+        return x
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    prev = torch.empty_like(ids)
+    first = torch.zeros_like(ids, dtype=torch.bool)
+    for b in range(len(sl)):
+        s, e = cu[b], cu[b + 1]
+        if e == s:
+            continue
+        prev[s + 1:e] = ids[s:e - 1]
+        if st[b] == 0:
+            prev[s] = 0
+            first[s] = True
+        else:
+            prev[s] = tok_state[sl[b]].long()
+        tok_state[sl[b]] = ids[e - 1].to(tok_state.dtype)
+    row = (prev * mul_prev + ids * mul_cur) % buckets
+    row = torch.where(first, torch.full_like(row, buckets), row)
+    return x + bigram[row].float()
+
+
+def group_norm_pair(x, a, b, w1, w2, groups, eps, out_dtype):
+    """x (fp32, in place) += a + b (either may be None); returns
+    (gnorm(x) * w1, gnorm(x) * w2) in out_dtype, where gnorm divides each of
+    ``groups`` equal runs of the row by its own root mean square. w2 None ->
+    second result None."""
+    if a is not None:
+        x.add_(a.float() if b is None else a.float() + b.float())
+    T, W = x.shape
+    xg = x.view(T, groups, W // groups)
+    n = (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, W)
+    h1 = (n * w1.float()).to(out_dtype)
+    h2 = (n * w2.float()).to(out_dtype) if w2 is not None else None
+    return h1, h2
+
+
+def cast_concat(x, x0, a, b, out_dtype):
+    """x (fp32, in place) += a + b (either may be None); returns [x | x0] in
+    out_dtype, [T, 2W]."""
+    if a is not None:
+        x.add_(a.float() if b is None else a.float() + b.float())
+    return torch.cat([x, x0], -1).to(out_dtype)
+
+
+def qk_norm_store(q, k, v, wq, wk, eps, k_cache, v_cache, slot_mapping) -> None:
+    """RMS norm over the head dim of q [T,H,D] (in place) and k [T,G,D] with
+    weights wq / wk [D]; the normed k and v go to the paged caches."""
+    def n(t, w):
+        tf = t.float()
+        return tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+
+    BS = k_cache.shape[2]
+    blk, off = slot_mapping // BS, slot_mapping % BS
+    k_cache[blk, :, off, :] = n(k, wk).to(k_cache.dtype)
+    v_cache[blk, :, off, :] = v.to(v_cache.dtype)
+    q.copy_(n(q, wq).to(q.dtype))
+
+
+def attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale, mask_kind,
+                      mask_size, keep_first, sink, gate=None, out_dtype=None) -> torch.Tensor:
+    """Softmax attention of packed query rows against the paged cache. Row t
+    at position p sees key j <= p of its own sequence when
+      mask_kind 0 (aligned blocks): floor(j / mask_size) == floor(p / mask_size)
+      mask_kind 1 (sliding window): p - j < mask_size or j < keep_first
+    (mask_size 0 = plain causal). ``sink``: one more term exp(0) in the
+    denominator. ``gate`` logits [T, H] (per head) or [T, H*Dv] (per element)."""
+    T, H, D = q.shape
+    _, G, BS, Dv = v_cache.shape
+    rep = H // G
+    out = torch.empty(T, H, Dv, dtype=out_dtype or q.dtype, device=q.device)
+    pos = positions.tolist()
+    seg = token_seg.tolist()
+    for t in range(T):
+        p = pos[t]
+        if mask_size <= 0:
+            idx = torch.arange(0, p + 1, device=q.device)
+        elif mask_kind == 0:
+            idx = torch.arange((p // mask_size) * mask_size, p + 1, device=q.device)
+        else:
+            lo = max(0, p - mask_size + 1)
+            idx = torch.cat([torch.arange(0, min(keep_first, lo), device=q.device),
+                             torch.arange(lo, p + 1, device=q.device)])
+        blocks = block_tables[seg[t]].long()[idx // BS]
+        kk = k_cache[blocks, :, idx % BS, :].float()
+        vv = v_cache[blocks, :, idx % BS, :].float()
+        qt = q[t].float().view(G, rep, D)
+        s = torch.einsum("grd,ngd->grn", qt, kk) * scale
+        if sink:
+            mx = s.max(-1, keepdim=True).values.clamp(min=0.0)
+            e = torch.exp(s - mx)
+            pr = e / (e.sum(-1, keepdim=True) + torch.exp(-mx))
+        else:
+            pr = torch.softmax(s, dim=-1)
+        o = torch.einsum("grn,ngd->grd", pr, vv).reshape(H, Dv)
+        if gate is not None:
+            gt = torch.sigmoid(gate[t].float())
+            o = o * (gt[:, None] if gt.numel() == H else gt.view(H, Dv))
+        out[t] = o.to(out.dtype)
+    return out
+
+
+def token_shift_mix(h, mu, shift_state, state_slots, cu_seqlens, seg_start, n_act, out_dtype):
+    """Mixes of each row with its predecessor: out[s] = h + (h_prev - h) * mu[s]
+    for the rows of mu [n, W]. The predecessor of a segment's first row is
+    shift_state[slot] (zeros for a fresh sequence); shift_state is set to the
+    segment's last row. Returns ([n_act, T, W] in out_dtype, [n - n_act, T, W]
+    fp32): the last mixes feed fp32 paths."""
+    T, W = h.shape
+    hf = h.float()
+    prev = torch.zeros_like(hf)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    for b in range(len(sl)):
+        s, e = cu[b], cu[b + 1]
+        if e == s:
+            continue
+        prev[s + 1:e] = hf[s:e - 1]
+        if st[b] > 0:
+            prev[s] = shift_state[sl[b]].float()
+        shift_state[sl[b]] = h[e - 1].to(shift_state.dtype)
+    mixes = hf[None] + (prev - hf)[None] * mu.float()[:, None, :]
+    return mixes[:n_act].to(out_dtype), mixes[n_act:].contiguous()
+
+
+def wkv_recurrence(r, k, v, d, w0, u, state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
+    """r, k, v [T,H,D|V]; d [T, H*D] fp32 decay pre-activation (w0 [H*D] is
+    added here), w = exp(-exp(d + w0)); u [H, D] bonus; state [slots,H,D,V]
+    fp32. Per head o_t = (S + diag(u) k v^T)^T r, then S <- diag(w) S + k v^T.
+    Returns o [T,H,V] fp32."""
+    T, H, D = r.shape
+    V = v.shape[2]
+    rf, kf, vf = r.float(), k.float(), v.float()
+    w = torch.exp(-torch.exp(d.float() + w0.float())).view(T, H, D)
+    uf = u.float()
+    o = torch.empty(T, H, V, dtype=torch.float32, device=r.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    for b in range(len(sl)):
+        S = state[sl[b]].clone() if st[b] > 0 else torch.zeros_like(state[sl[b]])
+        for t in range(cu[b], cu[b + 1]):
+            kv = kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S + uf.unsqueeze(-1) * kv, rf[t])
+            S = w[t].unsqueeze(-1) * S + kv
+        state[sl[b]] = S
+    return o
+
+
+def mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens, seg_start):
+    """q, k [T,H,D], v [T,H,V]; gates [T, 2H] fp32 (input | forget
+    pre-activations, gate_bias [2H] added here). i = cap tanh(./cap),
+    f = logsigmoid(cap tanh(./cap)); m_t = max(f + m, i), m starting at 0;
+    S <- e^(f+m-m_t) S + e^(i-m_t) k v^T, n likewise with k alone;
+    o = S^T q' / (max(|n . q'|, e^-m_t) + 1e-6), q' = q D^-1/2.
+    state [slots, H, D+1, V+1] fp32: [:, :, :D, :V] = S, [:, :, :D, V] = n,
+    [:, :, D, :] = m. Returns o [T,H,V] fp32."""
+    T, H, D = q.shape
+    V = v.shape[2]
+    qf, kf, vf = q.float() * (D ** -0.5), k.float(), v.float()
+    g = gates.float() + gate_bias.float()
+    ig = cap * torch.tanh(g[:, :H] / cap)
+    fg = torch.nn.functional.logsigmoid(cap * torch.tanh(g[:, H:] / cap))
+    o = torch.empty(T, H, V, dtype=torch.float32, device=q.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    ones = torch.ones(H, 1, dtype=torch.float32, device=q.device)
+    for b in range(len(sl)):
+        if st[b] > 0:
+            S = state[sl[b], :, :D, :].clone()             # [H, D, V+1], last column = n
+            m = state[sl[b], :, D, 0].clone()
+        else:
+            S = torch.zeros(H, D, V + 1, dtype=torch.float32, device=q.device)
+            m = torch.zeros(H, dtype=torch.float32, device=q.device)
+        for t in range(cu[b], cu[b + 1]):
+            m_new = torch.maximum(fg[t] + m, ig[t])
+            fa, fi = torch.exp(fg[t] + m - m_new), torch.exp(ig[t] - m_new)
+            ve = torch.cat([vf[t], ones], -1)
+            S = fa.view(H, 1, 1) * S + fi.view(H, 1, 1) * kf[t].unsqueeze(-1) * ve.unsqueeze(-2)
+            m = m_new
+            oe = torch.einsum("hdv,hd->hv", S, qf[t])
+            den = torch.maximum(oe[:, V].abs(), torch.exp(-m)) + 1e-6
+            o[t] = oe[:, :V] / den[:, None]
+        state[sl[b], :, :D, :] = S
+        state[sl[b], :, D, :] = m[:, None]
+    return o
+
+
+def head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype) -> torch.Tensor:
+    """o [T,H,S] fp32: each head is divided by its root mean square, the
+    concatenation is scaled by weight [H*S] and by the gate ([T, H*S]):
+    gate_act 'sigmoid' or 'silu' applied to the gate's logits."""
+    T, H, S = o.shape
+    y = (o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)).reshape(T, H * S) * weight.float()
+    gf = gate.float()
+    gf = torch.sigmoid(gf) if gate_act == "sigmoid" else torch.nn.functional.silu(gf)
+    return (y * gf).to(out_dtype)
+
+
+def gated_act(gate, up, limit: float, alpha: float, up_bias: float) -> torch.Tensor:
+    """min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + up_bias);
+    limit = inf, alpha = 1, up_bias = 0 is silu(g) * u."""
+    g = gate.float().clamp(max=limit)
+    u = up.float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + up_bias)).to(gate.dtype)
+
+
+def moe_route(z, correction, top, group_count, group_keep):
+    """z [T, N] fp32 router logits. Scores s = softmax(z); the choice is made
+    on c = s + correction among the experts of the ``group_keep`` groups (of
+    ``group_count`` equal runs of neighbours) whose largest c is largest;
+    ties go to the lower index. Returns (idx [T, top] int32, w [T, top] fp32
+    = chosen s / (their sum + 1e-20))."""
+    T, N = z.shape
+    s = torch.softmax(z.float(), -1)
+    c = s + correction.float()
+    per = N // group_count
+    gs = c.view(T, group_count, per).max(-1).values
+    # stable descending order = ties to the lower index
+    gord = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :group_keep]
+    gmask = torch.zeros(T, group_count, dtype=torch.bool, device=z.device)
+    gmask.scatter_(1, gord, True)
+    cm = torch.where(gmask.repeat_interleave(per, dim=1), c, torch.full_like(c, float("-inf")))
+    idx = torch.sort(cm, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = s.gather(1, idx)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.to(torch.int32), w
+
+
+def moe_combine(rows, h, rowidx, w, out_dtype) -> torch.Tensor:
+    """out[t] = sum_j w[t, j] * (rows[rowidx[t, j]] if rowidx >= 0 else h[t]),
+    summed in the order j = 0, 1, ... in fp32. rows [R, W], h [T, W]."""
+    T, top = rowidx.shape
+    out = torch.zeros(T, h.shape[1], dtype=torch.float32, device=h.device)
+    hf = h.float()
+    for j in range(top):
+        ri = rowidx[:, j].long()
+        src = torch.where((ri >= 0)[:, None], rows[ri.clamp(min=0)].float(), hf)
+        out += w[:, j:j + 1].float() * src
+    return out.to(out_dtype)
