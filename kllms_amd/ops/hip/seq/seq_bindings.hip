@@ -14,13 +14,35 @@ void seq_launch_sandwich_residual(float*, const void*, const void*, const float*
                                   const float*, void*, int, int, float, int, hipStream_t);
 void seq_launch_gated_rmsnorm(void*, const float*, const float*, const void*, int, int, int, int, float, int,
                               hipStream_t);
-void seq_launch_clamped_glu(void*, const void*, const void*, int64_t, int, int, float, float, int, hipStream_t);
+void seq_launch_gated_act(void*, const void*, const void*, int64_t, int, int, float, float, float, int,
+                          hipStream_t);
 void seq_launch_rope_pairs_store(void*, const void*, const void*, const int64_t*, const float*, void*, void*,
                                  const int64_t*, void*, int, int, int, int, int, int, int, int, int, int, int,
                                  hipStream_t);
-void seq_launch_attn_blocklocal_paged(void*, const void*, const void*, const void*, const int*, const int*,
-                                      const int64_t*, const void*, const int*, int, float, int, int, int, int,
-                                      int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_attn_masked_paged(void*, const void*, const void*, const void*, const int*, const int*,
+                                  const int64_t*, const void*, const int*, int, float, int, int, int, int, int,
+                                  int, int, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_qk_norm_store(void*, const void*, const void*, const float*, const float*, float, void*, void*,
+                              const int64_t*, int, int, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_embed_bigram(float*, const int64_t*, const void*, const void*, float, int, int, int, int*,
+                             const int*, const int*, const int*, const int*, int, int, int, int, hipStream_t);
+void seq_launch_group_norm_pair(float*, const void*, const void*, const float*, const float*, void*, void*, int,
+                                int, int, float, int, hipStream_t);
+void seq_launch_cast_concat(void*, float*, const float*, const void*, const void*, int, int, int, hipStream_t);
+void seq_launch_head_rmsnorm_gate(void*, const float*, const float*, const void*, int, int, int, int, float, int,
+                                  int, hipStream_t);
+void seq_launch_token_shift_mix(void*, float*, const void*, const float*, void*, const int*, const int*,
+                                const int*, const int*, int, int, int, int, int, int, hipStream_t);
+void seq_launch_moe_route(int*, float*, const float*, const float*, int, int, int, int, int, hipStream_t);
+void seq_launch_moe_combine(void*, const void*, const void*, const int*, const float*, int, int, int, int,
+                            hipStream_t);
+void seq_launch_wkv_recurrence(float*, const void*, const void*, const void*, const float*, const float*,
+                               const float*, float*, float*, float*, float*, float*, float*, const int*,
+                               const int*, const int*, int, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_mlstm_recurrence(float*, const void*, const void*, const void*, const float*, const float*, float,
+                                 float*, float*, float*, float*, float*, float*, float*, float*, const int*,
+                                 const int*, const int*, int, int, int, int, int, int, int, int, int,
+                                 hipStream_t);
 void seq_launch_head_gate(void*, const void*, int, int, int, int, int, hipStream_t);
 void seq_launch_linear_attn_decay(float*, const void*, const void*, const void*, const float*, float*, float*,
                                   const int*, const int*, const int*, int, int, int, int, int, int, int, int,
@@ -114,13 +136,15 @@ void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::T
                            (int)gate.stride(0), (float)eps, f32flag(out), cur_stream());
 }
 
-void clamped_glu(torch::Tensor out, torch::Tensor gate, torch::Tensor up, double limit, double alpha) {
+void gated_act(torch::Tensor out, torch::Tensor gate, torch::Tensor up, double limit, double alpha,
+               double up_bias) {
   CHECK_ACT(out); CHECK_ACT(gate); CHECK_SAME(up, gate); CHECK_SAME(out, gate); CHECK_ROWS2(gate); CHECK_ROWS2(up);
   TORCH_CHECK(up.is_cuda() && up.sizes() == gate.sizes() && up.stride(0) == gate.stride(0));
   TORCH_CHECK(out.is_contiguous() && out.numel() == gate.numel());
   if (gate.numel() == 0) return;
-  seq_launch_clamped_glu(out.data_ptr(), gate.data_ptr(), up.data_ptr(), gate.size(0), (int)gate.size(1),
-                         (int)gate.stride(0), (float)limit, (float)alpha, f32flag(gate), cur_stream());
+  seq_launch_gated_act(out.data_ptr(), gate.data_ptr(), up.data_ptr(), gate.size(0), (int)gate.size(1),
+                       (int)gate.stride(0), (float)limit, (float)alpha, (float)up_bias, f32flag(gate),
+                       cur_stream());
 }
 
 // caches: [NB, G, BS, D] / [NB, G, BS, Dv]; v: empty = store the un-rotated key as the value
@@ -159,32 +183,56 @@ void rope_pairs_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::
                               cur_stream());
 }
 
-void attn_blocklocal_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
-                           torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
-                           torch::Tensor gate, double scale, int64_t mask_size, torch::Tensor row_map) {
+// gate: empty, [T, H] (one logit per head) or [T, H*Dv] (one per output element)
+void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
+                       torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
+                       torch::Tensor gate, double scale, int64_t mask_kind, int64_t mask_size,
+                       int64_t keep_first, bool sink, torch::Tensor row_map) {
   CHECK_ACT(q); CHECK_ROWS3(q); CHECK_SAME(out, q); CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q);
   CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && k_cache.is_cuda() && v_cache.is_cuda() &&
               k_cache.is_contiguous() && v_cache.is_contiguous() && block_tables.dim() == 2);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   const int G = k_cache.size(1), BS = k_cache.size(2), Dv = v_cache.size(3);
-  TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && Dv <= 512 && mask_size >= 0);
+  TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && Dv <= 512 && mask_size >= 0 && keep_first >= 0);
+  TORCH_CHECK(mask_kind == 0 || mask_kind == 1, "mask_kind: 0 = aligned blocks, 1 = sliding window");
   TORCH_CHECK(out.numel() == (int64_t)T * H * Dv && token_seg.numel() == T && positions.numel() == T);
-  const bool has_gate = gate.numel() > 0;
-  if (has_gate) {
+  int gate_kind = 0;
+  if (gate.numel() > 0) {
     CHECK_ROWS2(gate); CHECK_SAME(gate, q);
-    TORCH_CHECK(gate.is_cuda() && gate.size(0) == T && gate.size(1) == H);
+    TORCH_CHECK(gate.is_cuda() && gate.size(0) == T && (gate.size(1) == H || gate.size(1) == (int64_t)H * Dv));
+    gate_kind = (gate.size(1) == (int64_t)H * Dv && Dv > 1) ? 2 : 1;
   }
   const bool mapped = row_map.numel() > 0;
   if (mapped) { CHECK_I32C(row_map); TORCH_CHECK(row_map.numel() <= T); }
   if (T == 0) return;
-  seq_launch_attn_blocklocal_paged(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                   block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
-                                   positions.data_ptr<int64_t>(), has_gate ? gate.data_ptr() : nullptr,
-                                   mapped ? row_map.data_ptr<int>() : nullptr, (int)row_map.numel(),
-                                   (float)scale, (int)mask_size, T, H, G, D, Dv, BS,
-                                   (int)block_tables.stride(0), (int)q.stride(0),
-                                   has_gate ? (int)gate.stride(0) : 0, f32flag(q), cur_stream());
+  seq_launch_attn_masked_paged(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                               block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
+                               positions.data_ptr<int64_t>(), gate_kind ? gate.data_ptr() : nullptr,
+                               mapped ? row_map.data_ptr<int>() : nullptr, (int)row_map.numel(),
+                               (float)scale, (int)mask_kind, (int)mask_size, (int)keep_first, sink ? 1 : 0,
+                               gate_kind, T, H, G, D, Dv, BS,
+                               (int)block_tables.stride(0), (int)q.stride(0),
+                               gate_kind ? (int)gate.stride(0) : 0, f32flag(q), cur_stream());
+}
+
+void qk_norm_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor wq, torch::Tensor wk,
+                   double eps, torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor slots) {
+  CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q);
+  CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q); CHECK_F32C(wq); CHECK_F32C(wk); CHECK_I64C(slots);
+  TORCH_CHECK(k.is_cuda() && v.is_cuda() && k_cache.is_cuda() && v_cache.is_cuda() && k_cache.is_contiguous() &&
+              v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
+  const int T = q.size(0), H = q.size(1), D = q.size(2), G = k.size(1);
+  const int BS = k_cache.size(2), Dv = v_cache.size(3);
+  TORCH_CHECK(k.size(0) == T && k.size(2) == D && v.size(0) == T && v.size(1) == G && v.size(2) == Dv);
+  TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(2) == BS &&
+              v_cache.size(0) == k_cache.size(0));
+  TORCH_CHECK(wq.numel() == D && wk.numel() == D && slots.numel() == T);
+  if (T == 0) return;
+  seq_launch_qk_norm_store(q.data_ptr(), k.data_ptr(), v.data_ptr(), wq.data_ptr<float>(), wk.data_ptr<float>(),
+                           (float)eps, k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr<int64_t>(), T, H,
+                           G, D, Dv, BS, (int)q.stride(0), (int)k.stride(0), (int)v.stride(0), f32flag(q),
+                           cur_stream());
 }
 
 void head_gate(torch::Tensor out, torch::Tensor gate) {
@@ -295,14 +343,201 @@ void gated_delta_rule(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::
                               f32flag(q), cur_stream());
 }
 
+// ---- parallel-layer family ------------------------------------------------------
+
+static void check_segments(const torch::Tensor& slots, const torch::Tensor& cu, const torch::Tensor& seg_start,
+                           int T) {
+  CHECK_I32C(slots); CHECK_I32C(cu); CHECK_I32C(seg_start);
+  TORCH_CHECK(cu.numel() == slots.numel() + 1 && seg_start.numel() == slots.numel());
+}
+
+void embed_bigram(torch::Tensor out, torch::Tensor ids, torch::Tensor table, torch::Tensor bigram, double scale,
+                  int64_t mul_prev, int64_t mul_cur, int64_t buckets, torch::Tensor tok_state,
+                  torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start, torch::Tensor token_seg) {
+  CHECK_F32C(out); CHECK_I64C(ids); CHECK_ACT(table);
+  TORCH_CHECK(table.is_contiguous() && table.dim() == 2);
+  const int T = ids.numel(), W = table.size(1), B = slots.numel();
+  TORCH_CHECK(out.numel() == (int64_t)T * W);
+  check_segments(slots, cu, seg_start, T);
+  CHECK_I32C(token_seg);
+  TORCH_CHECK(token_seg.numel() == T);
+  const bool has = bigram.numel() > 0;
+  if (has) {
+    CHECK_ACT(bigram); CHECK_SAME(bigram, table); CHECK_I32C(tok_state);
+    TORCH_CHECK(bigram.is_contiguous() && bigram.dim() == 2 && bigram.size(1) == W && buckets >= 1 &&
+                bigram.size(0) == buckets + 1);
+  }
+  if (T == 0) return;
+  seq_launch_embed_bigram(out.data_ptr<float>(), ids.data_ptr<int64_t>(), table.data_ptr(),
+                          has ? bigram.data_ptr() : nullptr, (float)scale, (int)mul_prev, (int)mul_cur,
+                          (int)buckets, has ? tok_state.data_ptr<int>() : nullptr, slots.data_ptr<int>(),
+                          cu.data_ptr<int>(), seg_start.data_ptr<int>(), token_seg.data_ptr<int>(), T, B, W,
+                          f32flag(table), cur_stream());
+}
+
+void group_norm_pair(torch::Tensor x, torch::Tensor a, torch::Tensor b, torch::Tensor w1, torch::Tensor w2,
+                     torch::Tensor out1, torch::Tensor out2, int64_t groups, double eps) {
+  CHECK_F32C(x); CHECK_F32C(w1); CHECK_ACT(out1);
+  TORCH_CHECK(x.dim() == 2 && out1.is_contiguous() && out1.numel() == x.numel());
+  const int T = x.size(0), W = x.size(1);
+  TORCH_CHECK(groups >= 1 && W % groups == 0 && w1.numel() == W && W <= 32768 && groups <= 1024);
+  const bool has_a = a.numel() > 0, has_b = b.numel() > 0, two = out2.numel() > 0;
+  TORCH_CHECK(has_a || !has_b, "second branch without a first");
+  if (has_a) { CHECK_ACT(a); CHECK_SAME(a, out1); TORCH_CHECK(a.is_contiguous() && a.numel() == x.numel()); }
+  if (has_b) { CHECK_ACT(b); CHECK_SAME(b, out1); TORCH_CHECK(b.is_contiguous() && b.numel() == x.numel()); }
+  if (two) {
+    CHECK_ACT(out2); CHECK_SAME(out2, out1); CHECK_F32C(w2);
+    TORCH_CHECK(out2.is_contiguous() && out2.numel() == x.numel() && w2.numel() == W);
+  }
+  if (T == 0) return;
+  seq_launch_group_norm_pair(x.data_ptr<float>(), has_a ? a.data_ptr() : nullptr, has_b ? b.data_ptr() : nullptr,
+                             w1.data_ptr<float>(), two ? w2.data_ptr<float>() : nullptr, out1.data_ptr(),
+                             two ? out2.data_ptr() : nullptr, T, W, (int)groups, (float)eps, f32flag(out1),
+                             cur_stream());
+}
+
+void cast_concat(torch::Tensor out, torch::Tensor x, torch::Tensor x0, torch::Tensor a, torch::Tensor b) {
+  CHECK_ACT(out); CHECK_F32C(x); CHECK_F32C(x0);
+  TORCH_CHECK(x.dim() == 2 && x0.sizes() == x.sizes() && out.is_contiguous() && out.numel() == 2 * x.numel());
+  const int T = x.size(0), W = x.size(1);
+  const bool has_a = a.numel() > 0, has_b = b.numel() > 0;
+  TORCH_CHECK(has_a || !has_b, "second branch without a first");
+  if (has_a) { CHECK_ACT(a); CHECK_SAME(a, out); TORCH_CHECK(a.is_contiguous() && a.numel() == x.numel()); }
+  if (has_b) { CHECK_ACT(b); CHECK_SAME(b, out); TORCH_CHECK(b.is_contiguous() && b.numel() == x.numel()); }
+  if (T == 0) return;
+  seq_launch_cast_concat(out.data_ptr(), x.data_ptr<float>(), x0.data_ptr<float>(),
+                         has_a ? a.data_ptr() : nullptr, has_b ? b.data_ptr() : nullptr, T, W, f32flag(out),
+                         cur_stream());
+}
+
+void head_rmsnorm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::Tensor gate, double eps,
+                       int64_t gate_act) {
+  CHECK_ACT(out); CHECK_F32C(o); CHECK_F32C(w); CHECK_ACT(gate); CHECK_SAME(gate, out); CHECK_ROWS2(gate);
+  TORCH_CHECK(o.dim() == 3 && out.is_contiguous() && out.numel() == o.numel());
+  const int T = o.size(0), H = o.size(1), S = o.size(2);
+  TORCH_CHECK(w.numel() == (int64_t)H * S && gate.size(0) == T && gate.size(1) == (int64_t)H * S);
+  TORCH_CHECK(gate_act == 0 || gate_act == 1, "gate_act: 0 = sigmoid, 1 = silu");
+  if (T == 0) return;
+  seq_launch_head_rmsnorm_gate(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(), T, H,
+                               S, (int)gate.stride(0), (float)eps, (int)gate_act, f32flag(out), cur_stream());
+}
+
+void token_shift_mix(torch::Tensor act, torch::Tensor f32, torch::Tensor h, torch::Tensor mu,
+                     torch::Tensor shift_state, torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start,
+                     torch::Tensor token_seg) {
+  CHECK_ACT(h); CHECK_F32C(mu); CHECK_SAME(shift_state, h); CHECK_I32C(token_seg);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && mu.dim() == 2 && shift_state.is_cuda() &&
+              shift_state.is_contiguous() && shift_state.dim() == 2);
+  const int T = h.size(0), W = h.size(1), n = mu.size(0), B = slots.numel();
+  check_segments(slots, cu, seg_start, T);
+  TORCH_CHECK(mu.size(1) == W && shift_state.size(1) == W && token_seg.numel() == T);
+  const int n_act = act.numel() > 0 ? (int)act.size(0) : 0;
+  if (n_act > 0) { CHECK_ACT(act); CHECK_SAME(act, h); TORCH_CHECK(act.is_contiguous()); }
+  if (n - n_act > 0) { CHECK_F32C(f32); }
+  TORCH_CHECK(act.numel() == (int64_t)n_act * T * W && f32.numel() == (int64_t)(n - n_act) * T * W);
+  if (T == 0) return;
+  seq_launch_token_shift_mix(n_act ? act.data_ptr() : nullptr, n - n_act ? f32.data_ptr<float>() : nullptr,
+                             h.data_ptr(), mu.data_ptr<float>(), shift_state.data_ptr(), slots.data_ptr<int>(),
+                             cu.data_ptr<int>(), seg_start.data_ptr<int>(), token_seg.data_ptr<int>(), T, B, W,
+                             n, n_act, f32flag(h), cur_stream());
+}
+
+void moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor z, torch::Tensor corr, int64_t top, int64_t gc,
+               int64_t gk) {
+  CHECK_I32C(idx); CHECK_F32C(w); CHECK_F32C(z); CHECK_F32C(corr);
+  TORCH_CHECK(z.dim() == 2);
+  const int T = z.size(0), N = z.size(1);
+  TORCH_CHECK(N >= 1 && N <= 256, "the router kernel serves up to 256 outputs");
+  TORCH_CHECK(gc >= 1 && N % gc == 0 && gk >= 1 && gk <= gc && top >= 1 && top <= (N / gc) * gk && top <= 64);
+  TORCH_CHECK(corr.numel() == N && idx.numel() == (int64_t)T * top && w.numel() == (int64_t)T * top);
+  if (T == 0) return;
+  seq_launch_moe_route(idx.data_ptr<int>(), w.data_ptr<float>(), z.data_ptr<float>(), corr.data_ptr<float>(), T,
+                       N, (int)top, (int)gc, (int)gk, cur_stream());
+}
+
+void moe_combine(torch::Tensor out, torch::Tensor rows, torch::Tensor h, torch::Tensor rowidx, torch::Tensor w) {
+  CHECK_ACT(out); CHECK_ACT(rows); CHECK_ACT(h); CHECK_SAME(rows, out); CHECK_SAME(h, out);
+  CHECK_I32C(rowidx); CHECK_F32C(w);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && rows.dim() == 2 && rows.is_contiguous() && out.is_contiguous());
+  const int T = h.size(0), W = h.size(1), top = rowidx.size(1);
+  TORCH_CHECK(rows.size(1) == W && out.numel() == h.numel() && rowidx.dim() == 2 && rowidx.size(0) == T &&
+              w.numel() == rowidx.numel());
+  if (T == 0) return;
+  seq_launch_moe_combine(out.data_ptr(), rows.data_ptr(), h.data_ptr(), rowidx.data_ptr<int>(),
+                         w.data_ptr<float>(), T, W, top, f32flag(out), cur_stream());
+}
+
+void wkv_recurrence(torch::Tensor o, torch::Tensor r, torch::Tensor k, torch::Tensor v, torch::Tensor d,
+                    torch::Tensor w0, torch::Tensor u, torch::Tensor state, torch::Tensor slots, torch::Tensor cu,
+                    torch::Tensor seg_start) {
+  CHECK_F32C(o); CHECK_ACT(r); CHECK_ROWS3(r); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, r); CHECK_SAME(v, r);
+  CHECK_F32C(d); CHECK_F32C(w0); CHECK_F32C(u); CHECK_F32C(state);
+  TORCH_CHECK(k.is_cuda() && v.is_cuda());
+  const int T = r.size(0), H = r.size(1), D = r.size(2), V = v.size(2), B = slots.numel();
+  check_segments(slots, cu, seg_start, T);
+  TORCH_CHECK(k.size(0) == T && k.size(1) == H && k.size(2) == D && v.size(0) == T && v.size(1) == H);
+  TORCH_CHECK(D <= 256, "the recurrence keeps up to 256 state rows per head in registers");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == V);
+  TORCH_CHECK(d.numel() == (int64_t)T * H * D && w0.numel() == (int64_t)H * D && u.numel() == (int64_t)H * D &&
+              o.numel() == (int64_t)T * H * V);
+  if (T == 0 || B == 0) return;
+  auto f32 = torch::dtype(torch::kFloat).device(r.device());
+  auto rp = torch::empty({(int64_t)T, (int64_t)H * D}, f32), kp = torch::empty({(int64_t)T, (int64_t)H * D}, f32);
+  auto wp = torch::empty({(int64_t)T, (int64_t)H * D}, f32), vp = torch::empty({(int64_t)T, (int64_t)H * V}, f32);
+  auto bonus = torch::empty({(int64_t)T, (int64_t)H}, f32);
+  seq_launch_wkv_recurrence(o.data_ptr<float>(), r.data_ptr(), k.data_ptr(), v.data_ptr(), d.data_ptr<float>(),
+                            w0.data_ptr<float>(), u.data_ptr<float>(), rp.data_ptr<float>(), kp.data_ptr<float>(),
+                            wp.data_ptr<float>(), vp.data_ptr<float>(), bonus.data_ptr<float>(),
+                            state.data_ptr<float>(), slots.data_ptr<int>(), cu.data_ptr<int>(),
+                            seg_start.data_ptr<int>(), T, B, H, D, V, (int)r.stride(0), (int)k.stride(0),
+                            (int)v.stride(0), f32flag(r), cur_stream());
+}
+
+// state [slots, H, D+1, V+1]: the matrix, the normaliser as column V, the running maximum in row D
+void mlstm_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor z,
+                      torch::Tensor zb, double cap, torch::Tensor state, torch::Tensor slots, torch::Tensor cu,
+                      torch::Tensor seg_start) {
+  CHECK_F32C(o); CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q);
+  CHECK_F32C(z); CHECK_F32C(zb); CHECK_F32C(state);
+  TORCH_CHECK(k.is_cuda() && v.is_cuda());
+  const int T = q.size(0), H = q.size(1), D = q.size(2), V = v.size(2), B = slots.numel();
+  check_segments(slots, cu, seg_start, T);
+  TORCH_CHECK(k.size(0) == T && k.size(1) == H && k.size(2) == D && v.size(0) == T && v.size(1) == H);
+  TORCH_CHECK(D <= 256, "the recurrence keeps up to 256 state rows per head in registers");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D + 1 && state.size(3) == V + 1);
+  TORCH_CHECK(z.numel() == (int64_t)T * 2 * H && zb.numel() == 2 * H && o.numel() == (int64_t)T * H * V && cap > 0);
+  if (T == 0 || B == 0) return;
+  auto f32 = torch::dtype(torch::kFloat).device(q.device());
+  auto qp = torch::empty({(int64_t)T, (int64_t)H * D}, f32), kp = torch::empty({(int64_t)T, (int64_t)H * D}, f32);
+  auto vp = torch::empty({(int64_t)T, (int64_t)H * V}, f32), oe = torch::empty({(int64_t)T, (int64_t)H * (V + 1)}, f32);
+  auto ig = torch::empty({(int64_t)T, (int64_t)H}, f32), fg = torch::empty({(int64_t)T, (int64_t)H}, f32);
+  auto mt = torch::empty({(int64_t)T, (int64_t)H}, f32);
+  seq_launch_mlstm_recurrence(o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(), z.data_ptr<float>(),
+                              zb.data_ptr<float>(), (float)cap, qp.data_ptr<float>(), kp.data_ptr<float>(),
+                              vp.data_ptr<float>(), ig.data_ptr<float>(), fg.data_ptr<float>(),
+                              oe.data_ptr<float>(), mt.data_ptr<float>(), state.data_ptr<float>(),
+                              slots.data_ptr<int>(), cu.data_ptr<int>(), seg_start.data_ptr<int>(), T, B, H, D, V,
+                              (int)q.stride(0), (int)k.stride(0), (int)v.stride(0), f32flag(q), cur_stream());
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_rmsnorm", &embed_rmsnorm);
   m.def("rmsnorm_cast", &rmsnorm_cast);
   m.def("sandwich_residual", &sandwich_residual);
   m.def("gated_rmsnorm", &gated_rmsnorm);
-  m.def("clamped_glu", &clamped_glu);
+  m.def("gated_act", &gated_act);
   m.def("rope_pairs_store", &rope_pairs_store);
-  m.def("attn_blocklocal_paged", &attn_blocklocal_paged);
+  m.def("attn_masked_paged", &attn_masked_paged);
+  m.def("qk_norm_store", &qk_norm_store);
+  m.def("embed_bigram", &embed_bigram);
+  m.def("group_norm_pair", &group_norm_pair);
+  m.def("cast_concat", &cast_concat);
+  m.def("head_rmsnorm_gate", &head_rmsnorm_gate);
+  m.def("token_shift_mix", &token_shift_mix);
+  m.def("moe_route", &moe_route);
+  m.def("moe_combine", &moe_combine);
+  m.def("wkv_recurrence", &wkv_recurrence);
+  m.def("mlstm_recurrence", &mlstm_recurrence);
   m.def("head_gate", &head_gate);
   m.def("attn_varlen_mfma", &attn_varlen_mfma);
   m.def("linear_attn_decay", &linear_attn_decay);

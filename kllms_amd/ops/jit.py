@@ -35,7 +35,8 @@ EXTENSIONS = {
     "_C_seq": {
         "dir": os.path.join(HIP_DIR, "seq"),
         # the dense MFMA prefill kernel is shared with _C (one source, two modules)
-        "kernels": ["seq_norm.hip", "seq_attn.hip", "seq_recurrent.hip", "../attn_prefill.hip"],
+        "kernels": ["seq_norm.hip", "seq_attn.hip", "seq_recurrent.hip", "seq_parallel.hip", "seq_gated.hip",
+                    "../attn_prefill.hip"],
         "bindings": ["seq_bindings.hip"],
         "headers": ["seq_common.h"],
     },
