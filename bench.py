@@ -28,7 +28,8 @@ aggregate. ``--parallel tp`` instead shards ONE engine across all ranks
 and scheduler, other ranks follow in lockstep (parallel/serve.py).
 
 ``--compare-families`` is a separate, single-GPU measurement: prefill and
-decode token throughput of the Zutalix family (listed-layer hybrid) beside
+decode token throughput of the listed-layer hybrid families (Zutalix, Medilix;
+``--families`` picks) beside
 the dense Llama stack of the same width / depth / heads / ff, straight through
 LLMEngine.generate (random-init weights, synthetic token ids). It prints its
 own JSON line and leaves the default workload untouched.
@@ -170,7 +171,7 @@ def compare_families(args) -> None:
     B, P, N = args.batch or 16, args.prompt_len, args.max_new or 64
     rows = []
     for size in sizes:
-        for fam in ("llama", "zutalix"):
+        for fam in [f for f in args.families.split(",") if f]:
             name = f"{fam}-{size}" if f"{fam}-{size}" in MODEL_PRESETS else f"{size}-{fam}"
             kw = dict(model=name, device=device, seed=0, use_hip_graphs=device != "cpu" and not args.no_graphs,
                       max_seq_len=P + N + 64, max_batch_size=max(B, 8), enable_prefix_caching=False,
@@ -208,7 +209,9 @@ def compare_families(args) -> None:
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--compare-families", action="store_true",
-                    help="prefill/decode tok/s of the Zutalix family beside the dense Llama stack of equal shape")
+                    help="prefill/decode tok/s of the hybrid families beside the dense Llama stack of equal shape")
+    ap.add_argument("--families", type=str, default="llama,zutalix,medilix",
+                    help="--compare-families: model families to time, in order")
     ap.add_argument("--sizes", type=str, default="1b-l6,8b-l6", help="--compare-families: preset size suffixes")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)

@@ -191,7 +191,6 @@ def forward(tokens: List[int], weights: Dict[str, torch.Tensor], cfg: dict, retu
         spec = cfg["layers"][li]
         pre = f"l{li}."
         h1 = group_rms(x, _w(weights, pre + "norm1"), groups, eps)
-        h2 = group_rms(x, _w(weights, pre + "norm2"), groups, eps)
         kind = spec["type"]
         if kind == "attention":
             y = attention(h1, weights, pre + "mix.", spec["mixer"], eps)
@@ -203,6 +202,7 @@ def forward(tokens: List[int], weights: Dict[str, torch.Tensor], cfg: dict, retu
             raise ValueError(kind)
         mlp = spec.get("mlp")
         if mlp:
+            h2 = group_rms(x, _w(weights, pre + "norm2"), groups, eps)
             if mlp["kind"] == "dense":
                 y = y + dense_ff(h2, weights, pre + "mlp.", mlp)
             else:
@@ -212,3 +212,66 @@ def forward(tokens: List[int], weights: Dict[str, torch.Tensor], cfg: dict, retu
     hf = group_rms(x, _w(weights, "final.norm"), groups, eps)
     logits = hf @ _w(weights, "head").T
     return (logits, layers_out) if return_layers else logits
+
+
+def random_weights(cfg: dict, seed: int, decay_rank: int = 5) -> Dict[str, torch.Tensor]:
+    """Random checkpoint for a config (values rounded to bfloat16, as a
+    checkpoint stores them). Norm weights vary around 1, decays reach far
+    back, gate biases are away from 0 so that every term matters."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def rn(*shape, std=1.0, mean=0.0):
+        return (torch.randn(*shape, generator=g) * std + mean).bfloat16().float()
+
+    def mat(o, i, gain=1.0):
+        return rn(o, i, std=gain * i ** -0.5)
+
+    w = {"embed": rn(V, W), "final.norm": rn(W, std=0.1, mean=1.0), "head": mat(V, W)}
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    if bg:
+        w["bigram"] = rn(bg["buckets"] + 1, W, std=0.5)
+    if cfg.get("loop"):
+        w["loop.in"] = mat(W, 2 * W, gain=1.4)
+    for i, sp in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", sp["mixer"]
+        w[p + "norm1"] = rn(W, std=0.1, mean=1.0)
+        q = p + "mix."
+        if sp["type"] == "attention":
+            H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            w.update({q + "q": mat(H * D, W), q + "k": mat(G * D, W), q + "v": mat(G * Dv, W),
+                      q + "g": mat(H * Dv, W), q + "o": mat(W, H * Dv),
+                      q + "q.norm": rn(D, std=0.2, mean=1.0), q + "k.norm": rn(D, std=0.2, mean=1.0)})
+        elif sp["type"] == "wkv":
+            H, D = m["heads"], m["dim"]
+            for s in "rkvgw":
+                w[q + "mu." + s] = torch.rand(W, generator=g).bfloat16().float()
+            for s in "rkvg":
+                w[q + s] = mat(H * D, W)
+            w.update({q + "w1": mat(decay_rank, W), q + "w2": mat(H * D, decay_rank),
+                      q + "w0": rn(H * D, std=0.8, mean=-2.5), q + "u": rn(H, D, std=0.5),
+                      q + "norm": rn(H * D, std=0.1, mean=1.0), q + "o": mat(W, H * D)})
+        else:
+            H, D, Dv = m["heads"], m["dim"], m["vdim"]
+            w.update({q + "q": mat(H * D, W), q + "k": mat(H * D, W), q + "v": mat(H * Dv, W),
+                      q + "g": mat(H * Dv, W), q + "o": mat(W, H * Dv), q + "norm": rn(H * Dv, std=0.1, mean=1.0),
+                      q + "i": mat(H, W, gain=2.0), q + "i.b": rn(H, std=0.5),
+                      q + "f": mat(H, W, gain=2.0), q + "f.b": rn(H, std=0.5, mean=2.0)})
+        mlp = sp.get("mlp")
+        if not mlp:
+            continue
+        w[p + "norm2"] = rn(W, std=0.1, mean=1.0)
+        q = p + "mlp."
+        if mlp["kind"] == "dense":
+            w.update({q + "gate": mat(mlp["ff"], W, gain=2.0), q + "up": mat(mlp["ff"], W, gain=2.0),
+                      q + "down": mat(W, mlp["ff"])})
+        else:
+            r = mlp["router"]
+            n = r["experts"] + r.get("identity", 0)
+            w[q + "router"] = mat(n, W, gain=2.0)
+            w[q + "correction"] = rn(n, std=0.1, mean=-0.05)
+            ff = mlp["expert"]["ff"]
+            for e in range(r["experts"]):
+                w.update({f"{q}e{e}.gate": mat(ff, W, gain=1.5), f"{q}e{e}.up": mat(ff, W, gain=1.5),
+                          f"{q}e{e}.down": mat(W, ff)})
+    return w
