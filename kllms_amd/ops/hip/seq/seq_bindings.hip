@@ -380,7 +380,7 @@ void group_norm_pair(torch::Tensor x, torch::Tensor a, torch::Tensor b, torch::T
   CHECK_F32C(x); CHECK_F32C(w1); CHECK_ACT(out1);
   TORCH_CHECK(x.dim() == 2 && out1.is_contiguous() && out1.numel() == x.numel());
   const int T = x.size(0), W = x.size(1);
-  TORCH_CHECK(groups >= 1 && W % groups == 0 && w1.numel() == W && W <= 32768 && groups <= 1024);
+  TORCH_CHECK(groups >= 1 && W % groups == 0 && w1.numel() == W && W <= 15360 && groups <= 1024);
   const bool has_a = a.numel() > 0, has_b = b.numel() > 0, two = out2.numel() > 0;
   TORCH_CHECK(has_a || !has_b, "second branch without a first");
   if (has_a) { CHECK_ACT(a); CHECK_SAME(a, out1); TORCH_CHECK(a.is_contiguous() && a.numel() == x.numel()); }

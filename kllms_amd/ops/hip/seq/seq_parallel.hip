@@ -80,6 +80,72 @@ __global__ void group_norm_pair_kernel(float* __restrict__ x, const T* __restric
   }
 }
 
+// 8-wide form (W and W/groups multiples of 8, 16-byte aligned rows): every
+// thread keeps its chunks of the row in registers; the chunks' sums of squares
+// go through LDS, one wave at a time adds up the chunks of a group in a fixed
+// order, and each chunk is scaled by its group's factor. NC = chunks per thread.
+template <typename T, int NC>
+__global__ void group_norm_pair_v8_kernel(float* __restrict__ x, const T* __restrict__ a,
+                                          const T* __restrict__ b, const float* __restrict__ w1,
+                                          const float* __restrict__ w2, T* __restrict__ out1,
+                                          T* __restrict__ out2, int W, int groups, float eps) {
+  extern __shared__ float part[];         // [W/8] chunk sums | [groups] factors
+  const int nchunk = W / 8, cpg = nchunk / groups;
+  float* rinv = part + nchunk;
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, nw = blockDim.x / WAVE;
+  float v[NC][8];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int ch = threadIdx.x + c * blockDim.x;
+    if (ch < nchunk) {
+      ld8(x + t * W + ch * 8, v[c]);
+      if (a != nullptr) {
+        float u[8];
+        ld8(a + t * W + ch * 8, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[c][e] += u[e];
+        if (b != nullptr) {
+          ld8(b + t * W + ch * 8, u);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[c][e] += u[e];
+        }
+        st8(x + t * W + ch * 8, v[c]);
+      }
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
+      part[ch] = ss;
+    }
+  }
+  __syncthreads();
+  for (int g = wave; g < groups; g += nw) {
+    float ss = 0.f;
+    for (int i = lane; i < cpg; i += WAVE) ss += part[g * cpg + i];
+    ss = wave_sum(ss);
+    if (lane == 0) rinv[g] = 1.0f / sqrtf(ss / (float)(cpg * 8) + eps);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int ch = threadIdx.x + c * blockDim.x;
+    if (ch < nchunk) {
+      const float r = rinv[ch / cpg];
+      float ww[8], y[8];
+      ld8(w1 + ch * 8, ww);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = v[c][e] * r * ww[e];
+      st8(out1 + t * W + ch * 8, y);
+      if (out2 != nullptr) {
+        ld8(w2 + ch * 8, ww);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = v[c][e] * r * ww[e];
+        st8(out2 + t * W + ch * 8, y);
+      }
+    }
+  }
+}
+
 // ---- loop entry: x += a + b, out = [x | x0] in the activation type ---------------
 template <typename T>
 __global__ void cast_concat_kernel(T* __restrict__ out, float* __restrict__ x, const float* __restrict__ x0,
@@ -142,6 +208,39 @@ __global__ void token_shift_mix_kernel(T* __restrict__ act, float* __restrict__ 
       const float v = hv + d * mu[(int64_t)s * W + i];
       if (s < n_act) stf(act + ((int64_t)s * T_ + t) * W + i, v);
       else f32[((int64_t)(s - n_act) * T_ + t) * W + i] = v;
+    }
+  }
+}
+
+// 8-wide form: one chunk of 8 columns per thread and iteration
+template <typename T>
+__global__ void token_shift_mix_v8_kernel(T* __restrict__ act, float* __restrict__ f32, const T* __restrict__ h,
+                                          const float* __restrict__ mu, const T* __restrict__ shift_state,
+                                          const int* __restrict__ slots, const int* __restrict__ cu,
+                                          const int* __restrict__ seg_start, const int* __restrict__ token_seg,
+                                          int T_, int W, int n, int n_act) {
+  const int64_t t = blockIdx.x;
+  const int b = token_seg[t];
+  const bool first = t == cu[b];
+  const bool fresh = seg_start[b] == 0;
+  const T* prow = first ? shift_state + (int64_t)slots[b] * W : h + (t - 1) * W;
+  for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+    float hv[8], d[8], m[8], y[8];
+    ld8(h + t * W + i, hv);
+    if (first && fresh) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d[e] = -hv[e];
+    } else {
+      ld8(prow + i, d);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) d[e] -= hv[e];
+    }
+    for (int s = 0; s < n; ++s) {
+      ld8(mu + (int64_t)s * W + i, m);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] = hv[e] + d[e] * m[e];
+      if (s < n_act) st8(act + ((int64_t)s * T_ + t) * W + i, y);
+      else st8(f32 + ((int64_t)(s - n_act) * T_ + t) * W + i, y);
     }
   }
 }
@@ -252,6 +351,24 @@ extern "C" void seq_launch_embed_bigram(float* out, const int64_t* ids, const vo
 extern "C" void seq_launch_group_norm_pair(float* x, const void* a, const void* b, const float* w1,
                                            const float* w2, void* out1, void* out2, int T_, int W, int groups,
                                            float eps, int is_f32, hipStream_t st) {
+  const int nchunk = W / 8;
+  if (W % 8 == 0 && (W / groups) % 8 == 0 && nchunk <= 2048 && aligned16(x) && aligned16(w1) &&
+      aligned16(out1) && (a == nullptr || aligned16(a)) && (b == nullptr || aligned16(b)) &&
+      (out2 == nullptr || (aligned16(out2) && aligned16(w2)))) {
+    // one or two chunks per thread, whole waves
+    int threads = nchunk <= 256 ? (nchunk + WAVE - 1) / WAVE * WAVE : ((nchunk + 1) / 2 + WAVE - 1) / WAVE * WAVE;
+    const size_t lds8 = (size_t)(nchunk + groups) * sizeof(float);
+    if (nchunk <= 256) {
+      DISPATCH_T(is_f32, hipLaunchKernelGGL((group_norm_pair_v8_kernel<T, 1>), dim3(T_), dim3(threads), lds8, st,
+                                            x, (const T*)a, (const T*)b, w1, w2, (T*)out1, (T*)out2, W, groups,
+                                            eps);)
+    } else {
+      DISPATCH_T(is_f32, hipLaunchKernelGGL((group_norm_pair_v8_kernel<T, 2>), dim3(T_), dim3(threads), lds8, st,
+                                            x, (const T*)a, (const T*)b, w1, w2, (T*)out1, (T*)out2, W, groups,
+                                            eps);)
+    }
+    return;
+  }
   const size_t lds = (size_t)(W + groups) * sizeof(float);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(group_norm_pair_kernel<T>, dim3(T_), dim3(row_threads(W)), lds, st, x,
                                         (const T*)a, (const T*)b, w1, w2, (T*)out1, (T*)out2, W, groups, eps);)
@@ -274,8 +391,14 @@ extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h,
                                            void* shift_state, const int* slots, const int* cu,
                                            const int* seg_start, const int* token_seg, int T_, int B, int W,
                                            int n, int n_act, int is_f32, hipStream_t st) {
+  const bool v8 = W % 8 == 0 && aligned16(h) && aligned16(mu) && aligned16(shift_state) &&
+                  (act == nullptr || aligned16(act)) && (f32 == nullptr || aligned16(f32));
+  const int th8 = W / 8 >= 256 ? 256 : ((W / 8 + WAVE - 1) / WAVE * WAVE);
   DISPATCH_T(is_f32,
-             hipLaunchKernelGGL(token_shift_mix_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)act, f32,
+             if (v8) hipLaunchKernelGGL(token_shift_mix_v8_kernel<T>, dim3(T_), dim3(th8), 0, st, (T*)act, f32,
+                                        (const T*)h, mu, (const T*)shift_state, slots, cu, seg_start, token_seg, T_,
+                                        W, n, n_act);
+             else hipLaunchKernelGGL(token_shift_mix_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)act, f32,
                                 (const T*)h, mu, (const T*)shift_state, slots, cu, seg_start, token_seg, T_, W, n,
                                 n_act);
              hipLaunchKernelGGL(shift_state_update_kernel<T>, dim3(B), dim3(row_threads(W)), 0, st, (const T*)h,

@@ -51,7 +51,7 @@ def test_embed_bigram(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W,groups", [(48, 3), (320, 1), (1000, 4)])
+@pytest.mark.parametrize("W,groups", [(48, 3), (320, 1), (1000, 4), (2048, 2), (4096, 8), (36, 2)])
 def test_group_norm_pair_and_concat(dtype, W, groups):
     T = 7
     x = rnd(T, W, std=3.0)
@@ -118,8 +118,31 @@ def test_qk_norm_and_masked_attention(dtype, D, Dv, mask):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_token_shift(dtype):
-    W = 200
+@pytest.mark.parametrize("D,Dv", [(64, 64), (128, 128), (24, 40)])
+@pytest.mark.parametrize("mask", [(1, 300, 5, True), (1, 0, 0, True), (0, 512, 0, False), (1, 1024, 4, True)])
+def test_masked_attention_long_context(dtype, D, Dv, mask):
+    """More visible keys than one pass of the kernel's waves covers (256):
+    a window of 300 with kept tokens, plain causal over 1100, a block of 512,
+    and a window of 1024 that positions beyond it slide out of."""
+    kind, size, keep, sink = mask
+    H, G, BS = 4, 2, 16
+    lens, starts = [3, 2, 1], [298, 700, 1100]
+    cu, st, tseg = segments(lens, starts)
+    NB = 3 * 70 + 2
+    kc = rnd(NB, G, BS, D, dtype=dtype, std=0.5)
+    vc = rnd(NB, G, BS, Dv, dtype=dtype, seed=1)
+    bt = (torch.randperm(NB)[:210].to(torch.int32).view(3, 70)).to(DEV).contiguous()
+    pos = torch.tensor([p for n, s in zip(lens, starts) for p in range(s, s + n)], device=DEV)
+    q = rnd(sum(lens), H, D, dtype=dtype, seed=2)
+    gate = rnd(sum(lens), H * Dv, dtype=dtype, seed=3)
+    o = ops.attn_masked_paged(q, kc, vc, bt, tseg, pos, 0.2, kind, size, keep, sink, gate)
+    r = torch_ref.attn_masked_paged(q, kc, vc, bt, tseg, pos, 0.2, kind, size, keep, sink, gate)
+    close(o, r, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("W", [200, 2048, 36])
+def test_token_shift(dtype, W):
     cu, st, tseg = segments([4, 1, 6], [0, 3, 9])
     slots = torch.tensor([1, 3, 0], dtype=torch.int32, device=DEV)
     h = rnd(11, W, dtype=dtype)
