@@ -465,11 +465,11 @@ class MlstmMixer(nn.Module):
         y = self.inp(h)
         s = self.inp.split
         z = F.linear(h.float(), self.gates)
-        o = ops.mlstm_recurrence(s(y, "q").unflatten(1, (sp.heads, sp.dim)),
-                                 s(y, "k").unflatten(1, (sp.heads, sp.dim)),
-                                 s(y, "v").unflatten(1, (sp.heads, sp.vdim)), z, self.gate_bias, sp.gate_cap,
-                                 st.rec, batch.state_slots, batch.cu_seqlens, batch.seg_start)
-        r = ops.head_rmsnorm_gate(o, self.norm, s(y, "g"), self.eps, "sigmoid", self.o_proj.dtype)
+        r = ops.mlstm_mix_out(s(y, "q").unflatten(1, (sp.heads, sp.dim)),
+                              s(y, "k").unflatten(1, (sp.heads, sp.dim)),
+                              s(y, "v").unflatten(1, (sp.heads, sp.vdim)), z, self.gate_bias, sp.gate_cap,
+                              st.rec, batch.state_slots, batch.cu_seqlens, batch.seg_start, self.norm, s(y, "g"),
+                              self.eps, self.o_proj.dtype)
         return F.linear(r, self.o_proj)
 
     def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
@@ -510,14 +510,13 @@ class RoutedExperts(nn.Module):
         sp = self.spec
         T, W = h.shape
         E, top = sp.experts, sp.top
-        z = F.linear(h.float(), self.router)
-        idx, w = ops.moe_route(z, self.correction, top, sp.group_count, sp.group_keep)
-        if T <= 8 * E:
+        dense = T <= 8 * E
+        idx, w, rowidx = ops.moe_route_rows(h, self.router, self.correction, top, sp.group_count, sp.group_keep,
+                                            E, dense)
+        if dense:
             gu = torch.bmm(h.unsqueeze(0).expand(E, T, W), self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)
             act = ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]).view(E, T, sp.ff)
             rows = torch.bmm(act, self.w_down.transpose(1, 2)).view(E * T, W)
-            t_idx = torch.arange(T, dtype=torch.int32, device=h.device).unsqueeze(1)
-            rowidx = torch.where(idx < E, idx * T + t_idx, torch.full_like(idx, -1))
             return ops.moe_combine(rows, h, rowidx, w, h.dtype)
         flat = idx.reshape(-1).long().clamp(max=E)                # identity experts sort last
         order = torch.argsort(flat, stable=True)

@@ -470,28 +470,70 @@ def wkv_recurrence(r, k, v, d, w0, u, state, state_slots, cu_seqlens, seg_start)
 def mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens, seg_start):
     if _gpu(q):
         o = torch.empty((q.shape[0], q.shape[1], v.shape[2]), dtype=torch.float32, device=q.device)
+        e = _none(q, torch.float32)
         _seq().mlstm_recurrence(o, q, k, v, gates, gate_bias, float(cap), state, state_slots, cu_seqlens,
-                                seg_start)
+                                seg_start, e, e)
         return o
     return torch_ref.mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens,
                                       seg_start)
 
 
+def mlstm_mix_out(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens, seg_start, weight, gate, eps,
+                  out_dtype):
+    """mlstm_recurrence followed by head_rmsnorm_gate(sigmoid); on the GPU the
+    read-out's division happens inside the norm kernel."""
+    if _gpu(q):
+        T, H, V = q.shape[0], q.shape[1], v.shape[2]
+        oe = torch.empty((T, H, V + 1), dtype=torch.float32, device=q.device)
+        mt = torch.empty((T, H), dtype=torch.float32, device=q.device)
+        _seq().mlstm_recurrence(_none(q, torch.float32), q, k, v, gates, gate_bias, float(cap), state, state_slots,
+                                cu_seqlens, seg_start, oe, mt)
+        out = torch.empty((T, H * V), dtype=out_dtype, device=q.device)
+        _seq().head_rmsnorm_gate(out, oe, weight, gate, eps, 0, mt)
+        return out
+    o = torch_ref.mlstm_recurrence(q, k, v, gates, gate_bias, cap, state, state_slots, cu_seqlens, seg_start)
+    return torch_ref.head_rmsnorm_gate(o, weight, gate, eps, "sigmoid", out_dtype)
+
+
 def head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype):
     if _gpu(o):
         out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
-        _seq().head_rmsnorm_gate(out, o, weight, gate, eps, 0 if gate_act == "sigmoid" else 1)
+        _seq().head_rmsnorm_gate(out, o, weight, gate, eps, 0 if gate_act == "sigmoid" else 1,
+                                 _none(o, torch.float32))
         return out
     return torch_ref.head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype)
 
 
 def moe_route(z, correction, top, group_count, group_keep):
+    """Routing from fp32 logits z [T, N]: (idx [T, top] int32, w [T, top] fp32)."""
     if _gpu(z):
         idx = torch.empty((z.shape[0], top), dtype=torch.int32, device=z.device)
         w = torch.empty((z.shape[0], top), dtype=torch.float32, device=z.device)
-        _seq().moe_route(idx, w, z, correction, int(top), int(group_count), int(group_keep))
+        _seq().moe_route(idx, w, _none(z, torch.int32), z, _none(z), correction, int(top), int(group_count),
+                         int(group_keep), 0)
         return idx, w
     return torch_ref.moe_route(z, correction, top, group_count, group_keep)
+
+
+def moe_route_rows(h, router, correction, top, group_count, group_keep, experts, all_experts_form):
+    """Router GEMV in fp32 + routing in one kernel. Returns (idx, w, rowidx);
+    rowidx [T, top] (only when all_experts_form) addresses rows of the
+    all-experts output [experts * T, W]: choice * T + row, -1 = identity."""
+    T = h.shape[0]
+    if _gpu(h):
+        idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
+        w = torch.empty((T, top), dtype=torch.float32, device=h.device)
+        rowidx = torch.empty((T, top), dtype=torch.int32, device=h.device) if all_experts_form else None
+        _seq().moe_route(idx, w, rowidx if rowidx is not None else _none(h, torch.int32), h, router, correction,
+                         int(top), int(group_count), int(group_keep), int(experts))
+        return idx, w, rowidx
+    z = torch.nn.functional.linear(h.float(), router)
+    idx, w = torch_ref.moe_route(z, correction, top, group_count, group_keep)
+    rowidx = None
+    if all_experts_form:
+        t_idx = torch.arange(T, dtype=torch.int32, device=h.device).unsqueeze(1)
+        rowidx = torch.where(idx < experts, idx * T + t_idx, torch.full_like(idx, -1))
+    return idx, w, rowidx
 
 
 def moe_combine(rows, h, rowidx, w, out_dtype):

@@ -29,11 +29,12 @@ void seq_launch_embed_bigram(float*, const int64_t*, const void*, const void*, f
 void seq_launch_group_norm_pair(float*, const void*, const void*, const float*, const float*, void*, void*, int,
                                 int, int, float, int, hipStream_t);
 void seq_launch_cast_concat(void*, float*, const float*, const void*, const void*, int, int, int, hipStream_t);
-void seq_launch_head_rmsnorm_gate(void*, const float*, const float*, const void*, int, int, int, int, float, int,
-                                  int, hipStream_t);
+void seq_launch_head_rmsnorm_gate(void*, const float*, const float*, const void*, const float*, int, int, int,
+                                  int, float, int, int, hipStream_t);
 void seq_launch_token_shift_mix(void*, float*, const void*, const float*, void*, const int*, const int*,
                                 const int*, const int*, int, int, int, int, int, int, hipStream_t);
-void seq_launch_moe_route(int*, float*, const float*, const float*, int, int, int, int, int, hipStream_t);
+void seq_launch_moe_route(int*, float*, int*, const float*, const void*, const float*, const float*, int, int, int,
+                          int, int, int, int, int, hipStream_t);
 void seq_launch_moe_combine(void*, const void*, const void*, const int*, const float*, int, int, int, int,
                             hipStream_t);
 void seq_launch_wkv_recurrence(float*, const void*, const void*, const void*, const float*, const float*,
@@ -410,16 +411,21 @@ void cast_concat(torch::Tensor out, torch::Tensor x, torch::Tensor x0, torch::Te
                          cur_stream());
 }
 
+// mt: empty, or [T, H] running maxima — then o is [T, H, S + 1] with the normaliser as its last column
 void head_rmsnorm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::Tensor gate, double eps,
-                       int64_t gate_act) {
+                       int64_t gate_act, torch::Tensor mt) {
   CHECK_ACT(out); CHECK_F32C(o); CHECK_F32C(w); CHECK_ACT(gate); CHECK_SAME(gate, out); CHECK_ROWS2(gate);
-  TORCH_CHECK(o.dim() == 3 && out.is_contiguous() && out.numel() == o.numel());
-  const int T = o.size(0), H = o.size(1), S = o.size(2);
+  const bool ext = mt.numel() > 0;
+  TORCH_CHECK(o.dim() == 3 && out.is_contiguous());
+  const int T = o.size(0), H = o.size(1), S = (int)o.size(2) - (ext ? 1 : 0);
+  TORCH_CHECK(S >= 1 && out.numel() == (int64_t)T * H * S);
   TORCH_CHECK(w.numel() == (int64_t)H * S && gate.size(0) == T && gate.size(1) == (int64_t)H * S);
   TORCH_CHECK(gate_act == 0 || gate_act == 1, "gate_act: 0 = sigmoid, 1 = silu");
+  if (ext) { CHECK_F32C(mt); TORCH_CHECK(mt.numel() == (int64_t)T * H); }
   if (T == 0) return;
-  seq_launch_head_rmsnorm_gate(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(), T, H,
-                               S, (int)gate.stride(0), (float)eps, (int)gate_act, f32flag(out), cur_stream());
+  seq_launch_head_rmsnorm_gate(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(),
+                               ext ? mt.data_ptr<float>() : nullptr, T, H, S, (int)gate.stride(0), (float)eps,
+                               (int)gate_act, f32flag(out), cur_stream());
 }
 
 void token_shift_mix(torch::Tensor act, torch::Tensor f32, torch::Tensor h, torch::Tensor mu,
@@ -442,17 +448,33 @@ void token_shift_mix(torch::Tensor act, torch::Tensor f32, torch::Tensor h, torc
                              n, n_act, f32flag(h), cur_stream());
 }
 
-void moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor z, torch::Tensor corr, int64_t top, int64_t gc,
-               int64_t gk) {
-  CHECK_I32C(idx); CHECK_F32C(w); CHECK_F32C(z); CHECK_F32C(corr);
-  TORCH_CHECK(z.dim() == 2);
-  const int T = z.size(0), N = z.size(1);
+// x: fp32 logits [T, N] (router empty), or the rows h [T, W] with router [N, W] fp32 — then the logits are
+// computed in the kernel. rowidx: empty, or [T, top] for the all-experts form over `experts` real experts.
+void moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor rowidx, torch::Tensor x, torch::Tensor router,
+               torch::Tensor corr, int64_t top, int64_t gc, int64_t gk, int64_t experts) {
+  CHECK_I32C(idx); CHECK_F32C(w); CHECK_F32C(corr);
+  TORCH_CHECK(x.dim() == 2 && x.is_cuda() && x.is_contiguous());
+  const bool fused = router.numel() > 0;
+  const int T = x.size(0), N = corr.numel();
+  int W = 0;
+  if (fused) {
+    CHECK_ACT(x); CHECK_F32C(router);
+    W = x.size(1);
+    TORCH_CHECK(router.dim() == 2 && router.size(0) == N && router.size(1) == W);
+  } else {
+    CHECK_F32C(x);
+    TORCH_CHECK(x.size(1) == N);
+  }
   TORCH_CHECK(N >= 1 && N <= 256, "the router kernel serves up to 256 outputs");
   TORCH_CHECK(gc >= 1 && N % gc == 0 && gk >= 1 && gk <= gc && top >= 1 && top <= (N / gc) * gk && top <= 64);
-  TORCH_CHECK(corr.numel() == N && idx.numel() == (int64_t)T * top && w.numel() == (int64_t)T * top);
+  TORCH_CHECK(idx.numel() == (int64_t)T * top && w.numel() == (int64_t)T * top);
+  const bool rows = rowidx.numel() > 0;
+  if (rows) { CHECK_I32C(rowidx); TORCH_CHECK(rowidx.numel() == (int64_t)T * top && experts * T < (1LL << 31)); }
   if (T == 0) return;
-  seq_launch_moe_route(idx.data_ptr<int>(), w.data_ptr<float>(), z.data_ptr<float>(), corr.data_ptr<float>(), T,
-                       N, (int)top, (int)gc, (int)gk, cur_stream());
+  seq_launch_moe_route(idx.data_ptr<int>(), w.data_ptr<float>(), rows ? rowidx.data_ptr<int>() : nullptr,
+                       fused ? nullptr : x.data_ptr<float>(), fused ? x.data_ptr() : nullptr,
+                       fused ? router.data_ptr<float>() : nullptr, corr.data_ptr<float>(), T, N, W, (int)top,
+                       (int)gc, (int)gk, (int)experts, fused ? f32flag(x) : 1, cur_stream());
 }
 
 void moe_combine(torch::Tensor out, torch::Tensor rows, torch::Tensor h, torch::Tensor rowidx, torch::Tensor w) {
@@ -494,10 +516,14 @@ void wkv_recurrence(torch::Tensor o, torch::Tensor r, torch::Tensor k, torch::Te
 }
 
 // state [slots, H, D+1, V+1]: the matrix, the normaliser as column V, the running maximum in row D
+// o [T, H, V]: the read-out. With o empty, oe [T, H, V+1] (un-normalised read-out and normaliser) and
+// mt [T, H] (running maxima) are filled instead, for a norm kernel that divides on the way.
 void mlstm_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor z,
                       torch::Tensor zb, double cap, torch::Tensor state, torch::Tensor slots, torch::Tensor cu,
-                      torch::Tensor seg_start) {
-  CHECK_F32C(o); CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q);
+                      torch::Tensor seg_start, torch::Tensor oe, torch::Tensor mt) {
+  const bool raw = o.numel() == 0;
+  if (!raw) { CHECK_F32C(o); }
+  CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q);
   CHECK_F32C(z); CHECK_F32C(zb); CHECK_F32C(state);
   TORCH_CHECK(k.is_cuda() && v.is_cuda());
   const int T = q.size(0), H = q.size(1), D = q.size(2), V = v.size(2), B = slots.numel();
@@ -505,14 +531,21 @@ void mlstm_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::
   TORCH_CHECK(k.size(0) == T && k.size(1) == H && k.size(2) == D && v.size(0) == T && v.size(1) == H);
   TORCH_CHECK(D <= 256, "the recurrence keeps up to 256 state rows per head in registers");
   TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D + 1 && state.size(3) == V + 1);
-  TORCH_CHECK(z.numel() == (int64_t)T * 2 * H && zb.numel() == 2 * H && o.numel() == (int64_t)T * H * V && cap > 0);
-  if (T == 0 || B == 0) return;
+  TORCH_CHECK(z.numel() == (int64_t)T * 2 * H && zb.numel() == 2 * H && cap > 0);
+  TORCH_CHECK(raw || o.numel() == (int64_t)T * H * V);
   auto f32 = torch::dtype(torch::kFloat).device(q.device());
+  if (raw) {
+    CHECK_F32C(oe); CHECK_F32C(mt);
+    TORCH_CHECK(oe.numel() == (int64_t)T * H * (V + 1) && mt.numel() == (int64_t)T * H);
+  } else {
+    oe = torch::empty({(int64_t)T, (int64_t)H * (V + 1)}, f32);
+    mt = torch::empty({(int64_t)T, (int64_t)H}, f32);
+  }
+  if (T == 0 || B == 0) return;
   auto qp = torch::empty({(int64_t)T, (int64_t)H * D}, f32), kp = torch::empty({(int64_t)T, (int64_t)H * D}, f32);
-  auto vp = torch::empty({(int64_t)T, (int64_t)H * V}, f32), oe = torch::empty({(int64_t)T, (int64_t)H * (V + 1)}, f32);
+  auto vp = torch::empty({(int64_t)T, (int64_t)H * V}, f32);
   auto ig = torch::empty({(int64_t)T, (int64_t)H}, f32), fg = torch::empty({(int64_t)T, (int64_t)H}, f32);
-  auto mt = torch::empty({(int64_t)T, (int64_t)H}, f32);
-  seq_launch_mlstm_recurrence(o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(), z.data_ptr<float>(),
+  seq_launch_mlstm_recurrence(raw ? nullptr : o.data_ptr<float>(), q.data_ptr(), k.data_ptr(), v.data_ptr(), z.data_ptr<float>(),
                               zb.data_ptr<float>(), (float)cap, qp.data_ptr<float>(), kp.data_ptr<float>(),
                               vp.data_ptr<float>(), ig.data_ptr<float>(), fg.data_ptr<float>(),
                               oe.data_ptr<float>(), mt.data_ptr<float>(), state.data_ptr<float>(),

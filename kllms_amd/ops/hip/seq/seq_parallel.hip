@@ -165,18 +165,22 @@ __global__ void cast_concat_kernel(T* __restrict__ out, float* __restrict__ x, c
 
 // ---- per-head RMS norm, full-width weight, activated gate ------------------------
 // o [T, H, S] fp32; out[t, h*S + i] = o / rms(o[t,h,:]) * w[h*S + i] * act(gate[t, h*S + i]);
-// act = sigmoid (0) or silu (1). One wave per (row, head).
+// act = sigmoid (0) or silu (1). One wave per (row, head). With mt != nullptr the
+// head rows of o are S + 1 wide: the last entry is a normaliser n.q and the
+// head is first divided by max(|n.q|, e^-mt) + 1e-6 (the mlstm read-out).
 template <typename T>
 __global__ void head_rmsnorm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
-                                         const float* __restrict__ w, const T* __restrict__ gate, int H, int S,
+                                         const float* __restrict__ w, const T* __restrict__ gate,
+                                         const float* __restrict__ mt, int H, int S,
                                          int gate_stride, float eps, int gate_act) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y, lane = threadIdx.x;
-  const float* orow = o + (t * H + h) * S;
+  const float* orow = o + (t * H + h) * (mt != nullptr ? S + 1 : S);
+  const float pre = mt != nullptr ? 1.0f / (fmaxf(fabsf(orow[S]), expf(-mt[t * H + h])) + 1e-6f) : 1.0f;
   float ss = 0.f;
-  for (int i = lane; i < S; i += WAVE) { const float v = orow[i]; ss += v * v; }
+  for (int i = lane; i < S; i += WAVE) { const float v = orow[i] * pre; ss += v * v; }
   ss = wave_sum(ss);
-  const float r = 1.0f / sqrtf(ss / (float)S + eps);
+  const float r = pre / sqrtf(ss / (float)S + eps);
   const T* grow = gate + t * gate_stride + (int64_t)h * S;
   for (int i = lane; i < S; i += WAVE) {
     const float g = ldf(grow + i);
@@ -260,16 +264,36 @@ __global__ void shift_state_update_kernel(const T* __restrict__ h, T* __restrict
 // outputs form `gc` equal groups of neighbours, a group's score is its largest
 // c, the best `gk` groups stay eligible; the `top` eligible outputs with the
 // largest c are chosen (ties: the lower index). w = chosen s / (sum + 1e-20).
+// The logits come from z [T, N], or (z == nullptr) are computed here in fp32
+// as router [N, W] times the row of h. rowidx (optional) receives, for the
+// all-experts form with E real experts over T_ rows, choice * T_ + row for a
+// real expert and -1 for an identity expert.
 #define ROUTE_MAX_N 256
+template <typename T>
 __global__ void __launch_bounds__(WAVE) moe_route_kernel(int* __restrict__ idx, float* __restrict__ wout,
-                                                         const float* __restrict__ z,
-                                                         const float* __restrict__ corr, int N, int top, int gc,
-                                                         int gk) {
-  __shared__ float cs[ROUTE_MAX_N], ss[ROUTE_MAX_N], gmax[ROUTE_MAX_N];
+                                                         int* __restrict__ rowidx, const float* __restrict__ z,
+                                                         const T* __restrict__ h,
+                                                         const float* __restrict__ router,
+                                                         const float* __restrict__ corr, int N, int W, int top,
+                                                         int gc, int gk, int E, int T_) {
+  __shared__ float cs[ROUTE_MAX_N], ss[ROUTE_MAX_N], gmax[ROUTE_MAX_N], zs[ROUTE_MAX_N];
   __shared__ int ok[ROUTE_MAX_N];
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
-  const float* zr = z + t * N;
+  if (z != nullptr) {
+    for (int e = lane; e < N; e += WAVE) zs[e] = z[t * N + e];
+  } else {
+    const T* hr = h + t * W;
+    for (int e = 0; e < N; ++e) {
+      const float* rr = router + (int64_t)e * W;
+      float acc = 0.f;
+      for (int i = lane; i < W; i += WAVE) acc += ldf(hr + i) * rr[i];
+      acc = wave_sum(acc);
+      if (lane == 0) zs[e] = acc;
+    }
+  }
+  __syncthreads();
+  const float* zr = zs;
   float mx = -INFINITY;
   for (int e = lane; e < N; e += WAVE) mx = fmaxf(mx, zr[e]);
   mx = wave_max(mx);
@@ -311,7 +335,11 @@ __global__ void __launch_bounds__(WAVE) moe_route_kernel(int* __restrict__ idx, 
     const float sv = ss[bi];
     wsum += sv;
     if (lane == r) mine = sv;
-    if (lane == 0) { idx[t * top + r] = bi; cs[bi] = -INFINITY; }
+    if (lane == 0) {
+      idx[t * top + r] = bi;
+      if (rowidx != nullptr) rowidx[t * top + r] = bi < E ? bi * T_ + (int)t : -1;
+      cs[bi] = -INFINITY;
+    }
     __syncthreads();
   }
   if (lane < top) wout[t * top + lane] = mine / (wsum + 1e-20f);
@@ -381,10 +409,10 @@ extern "C" void seq_launch_cast_concat(void* out, float* x, const float* x0, con
 }
 
 extern "C" void seq_launch_head_rmsnorm_gate(void* out, const float* o, const float* w, const void* gate,
-                                             int T_, int H, int S, int gate_stride, float eps, int gate_act,
-                                             int is_f32, hipStream_t st) {
+                                             const float* mt, int T_, int H, int S, int gate_stride, float eps,
+                                             int gate_act, int is_f32, hipStream_t st) {
   DISPATCH_T(is_f32, hipLaunchKernelGGL(head_rmsnorm_gate_kernel<T>, dim3(T_, H), dim3(WAVE), 0, st, (T*)out, o,
-                                        w, (const T*)gate, H, S, gate_stride, eps, gate_act);)
+                                        w, (const T*)gate, mt, H, S, gate_stride, eps, gate_act);)
 }
 
 extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h, const float* mu,
@@ -405,9 +433,11 @@ extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h,
                                 (T*)shift_state, slots, cu, W);)
 }
 
-extern "C" void seq_launch_moe_route(int* idx, float* w, const float* z, const float* corr, int T_, int N,
-                                     int top, int gc, int gk, hipStream_t st) {
-  hipLaunchKernelGGL(moe_route_kernel, dim3(T_), dim3(WAVE), 0, st, idx, w, z, corr, N, top, gc, gk);
+extern "C" void seq_launch_moe_route(int* idx, float* w, int* rowidx, const float* z, const void* h,
+                                     const float* router, const float* corr, int T_, int N, int W, int top,
+                                     int gc, int gk, int E, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_route_kernel<T>, dim3(T_), dim3(WAVE), 0, st, idx, w, rowidx, z,
+                                        (const T*)h, router, corr, N, W, top, gc, gk, E, T_);)
 }
 
 extern "C" void seq_launch_moe_combine(void* out, const void* rows, const void* h, const int* rowidx,

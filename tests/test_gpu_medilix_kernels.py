@@ -228,3 +228,42 @@ def test_combine(dtype):
     rowidx = torch.randint(-1, R, (T, top), device=DEV, dtype=torch.int32)
     w = torch.rand(T, top, device=DEV)
     close(ops.moe_combine(rows, h, rowidx, w, dtype), torch_ref.moe_combine(rows, h, rowidx, w, dtype), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,E,top,gc,gk", [(12, 8, 3, 2, 1), (8, 8, 2, 1, 1), (9, 6, 2, 3, 2)])
+def test_router_with_its_projection(dtype, N, E, top, gc, gk):
+    """Router logits computed inside the routing kernel, and the row indices of
+    the all-experts form."""
+    T, W = 40, 200
+    h = rnd(T, W, dtype=dtype)
+    router = rnd(N, W, std=0.3, seed=1)
+    corr = rnd(N, seed=2) * 0.05
+    idx, w, rowidx = ops.moe_route_rows(h, router, corr, top, gc, gk, E, True)
+    z = torch.nn.functional.linear(h.float(), router)
+    ridx, rw = torch_ref.moe_route(z, corr, top, gc, gk)
+    assert torch.equal(idx, ridx)
+    close(w, rw, torch.float32, scale=5)
+    t_idx = torch.arange(T, dtype=torch.int32, device=DEV).unsqueeze(1)
+    assert torch.equal(rowidx, torch.where(ridx < E, ridx * T + t_idx, torch.full_like(ridx, -1)))
+    assert ops.moe_route_rows(h, router, corr, top, gc, gk, E, False)[2] is None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,D,V", [(2, 48, 64), (3, 16, 24)])
+def test_mlstm_with_fused_read_out(dtype, H, D, V):
+    lens, starts = [45, 1, 6], [0, 5, 77]
+    cu, st, _ = segments(lens, starts)
+    T = sum(lens)
+    slots = torch.tensor([3, 1, 0], dtype=torch.int32, device=DEV)
+    q, k, v = (rnd(T, H, D if s < 3 else V, dtype=dtype, std=0.7, seed=s) for s in (1, 2, 3))
+    z, zb = rnd(T, 2 * H, std=3.0, seed=4), rnd(2 * H, seed=5)
+    s1 = rnd(4, H, D + 1, V + 1, seed=7) * 0.3
+    s1[:, :, D, :] = torch.rand(4, H, 1, device=DEV) * 3
+    s2 = s1.clone()
+    wt = rnd(H * V, seed=8) * 0.1 + 1
+    gate = rnd(T, H * V, dtype=dtype, seed=9)
+    got = ops.mlstm_mix_out(q, k, v, z, zb, 15.0, s1, slots, cu, st, wt, gate, 1e-5, dtype)
+    o = torch_ref.mlstm_recurrence(q, k, v, z, zb, 15.0, s2, slots, cu, st)
+    close(got, torch_ref.head_rmsnorm_gate(o, wt, gate, 1e-5, "sigmoid", dtype), dtype)
+    close(s1, s2, torch.float32, scale=5)
