@@ -260,7 +260,7 @@ __global__ void shift_state_update_kernel(const T* __restrict__ h, T* __restrict
 }
 
 // ---- router --------------------------------------------------------------------
-// One wave per row. s = softmax(z) over the N outputs; c = s + correction; the
+// One workgroup per row (the routing proper is its first wave's). s = softmax(z) over the N outputs; c = s + correction; the
 // outputs form `gc` equal groups of neighbours, a group's score is its largest
 // c, the best `gk` groups stay eligible; the `top` eligible outputs with the
 // largest c are chosen (ties: the lower index). w = chosen s / (sum + 1e-20).
@@ -270,79 +270,96 @@ __global__ void shift_state_update_kernel(const T* __restrict__ h, T* __restrict
 // real expert and -1 for an identity expert.
 #define ROUTE_MAX_N 256
 template <typename T>
-__global__ void __launch_bounds__(WAVE) moe_route_kernel(int* __restrict__ idx, float* __restrict__ wout,
-                                                         int* __restrict__ rowidx, const float* __restrict__ z,
-                                                         const T* __restrict__ h,
-                                                         const float* __restrict__ router,
-                                                         const float* __restrict__ corr, int N, int W, int top,
-                                                         int gc, int gk, int E, int T_) {
+__global__ void __launch_bounds__(256) moe_route_kernel(int* __restrict__ idx, float* __restrict__ wout,
+                                                        int* __restrict__ rowidx, const float* __restrict__ z,
+                                                        const T* __restrict__ h,
+                                                        const float* __restrict__ router,
+                                                        const float* __restrict__ corr, int N, int W, int top,
+                                                        int gc, int gk, int E, int T_, int vec) {
   __shared__ float cs[ROUTE_MAX_N], ss[ROUTE_MAX_N], gmax[ROUTE_MAX_N], zs[ROUTE_MAX_N];
   __shared__ int ok[ROUTE_MAX_N];
   const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, nw = blockDim.x / WAVE;
+  // logits: every wave of the block takes outputs in turn; the routing proper is wave 0's
   if (z != nullptr) {
-    for (int e = lane; e < N; e += WAVE) zs[e] = z[t * N + e];
+    for (int e = threadIdx.x; e < N; e += blockDim.x) zs[e] = z[t * N + e];
   } else {
     const T* hr = h + t * W;
-    for (int e = 0; e < N; ++e) {
+    for (int e = wave; e < N; e += nw) {
       const float* rr = router + (int64_t)e * W;
       float acc = 0.f;
-      for (int i = lane; i < W; i += WAVE) acc += ldf(hr + i) * rr[i];
+      if (vec) {
+        for (int c = lane * 8; c < W; c += WAVE * 8) {
+          float hv[8], rv[8];
+          ld8(hr + c, hv);
+          ld8(rr + c, rv);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc += hv[k] * rv[k];
+        }
+      } else {
+        for (int i = lane; i < W; i += WAVE) acc += ldf(hr + i) * rr[i];
+      }
       acc = wave_sum(acc);
       if (lane == 0) zs[e] = acc;
     }
   }
   __syncthreads();
-  const float* zr = zs;
-  float mx = -INFINITY;
-  for (int e = lane; e < N; e += WAVE) mx = fmaxf(mx, zr[e]);
-  mx = wave_max(mx);
-  float sum = 0.f;
-  for (int e = lane; e < N; e += WAVE) { const float p = expf(zr[e] - mx); ss[e] = p; sum += p; }
-  sum = wave_sum(sum);
-  for (int e = lane; e < N; e += WAVE) { ss[e] /= sum; cs[e] = ss[e] + corr[e]; }
-  __syncthreads();
   const int per = N / gc;
-  for (int g = lane; g < gc; g += WAVE) {
-    float m = -INFINITY;
-    for (int i = 0; i < per; ++i) m = fmaxf(m, cs[g * per + i]);
-    gmax[g] = m;
-    ok[g] = 0;
+  if (wave == 0) {
+    float mx = -INFINITY;
+    for (int e = lane; e < N; e += WAVE) mx = fmaxf(mx, zs[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < N; e += WAVE) { const float p = expf(zs[e] - mx); ss[e] = p; sum += p; }
+    sum = wave_sum(sum);
+    for (int e = lane; e < N; e += WAVE) { ss[e] /= sum; cs[e] = ss[e] + corr[e]; }
   }
   __syncthreads();
-  if (lane == 0) {
+  if (wave == 0) {
+    for (int g = lane; g < gc; g += WAVE) {
+      float m = -INFINITY;
+      for (int i = 0; i < per; ++i) m = fmaxf(m, cs[g * per + i]);
+      gmax[g] = m;
+      ok[g] = 0;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
     for (int r = 0; r < gk; ++r) {
       int best = -1;
       for (int g = 0; g < gc; ++g)
         if (!ok[g] && (best < 0 || gmax[g] > gmax[best])) best = g;
-      ok[best] = 1;
+      if (best >= 0) ok[best] = 1;
     }
   }
   __syncthreads();
-  float wsum = 0.f, mine = 0.f;       // lane j keeps the j-th choice's score
+  float wsum = 0.f, mine = 0.f;       // lane j of wave 0 keeps the j-th choice's score
   for (int r = 0; r < top; ++r) {
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int e = lane; e < N; e += WAVE) {
-      if (ok[e / per] && (cs[e] > bv)) { bv = cs[e]; bi = e; }       // ascending e: ties keep the lower index
-    }
+    if (wave == 0) {
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int e = lane; e < N; e += WAVE) {
+        if (ok[e / per] && (cs[e] > bv)) { bv = cs[e]; bi = e; }     // ascending e: ties keep the lower index
+      }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float ov = __shfl_xor(bv, off);
-      const int oi = __shfl_xor(bi, off);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-    const float sv = ss[bi];
-    wsum += sv;
-    if (lane == r) mine = sv;
-    if (lane == 0) {
-      idx[t * top + r] = bi;
-      if (rowidx != nullptr) rowidx[t * top + r] = bi < E ? bi * T_ + (int)t : -1;
-      cs[bi] = -INFINITY;
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off);
+        const int oi = __shfl_xor(bi, off);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      if (bi >= N) bi = 0;             // nothing comparable left (not-a-number scores): stay in range
+      const float sv = ss[bi];
+      wsum += sv;
+      if (lane == r) mine = sv;
+      if (lane == 0) {
+        idx[t * top + r] = bi;
+        if (rowidx != nullptr) rowidx[t * top + r] = bi < E ? bi * T_ + (int)t : -1;
+        cs[bi] = -INFINITY;
+      }
     }
     __syncthreads();
   }
-  if (lane < top) wout[t * top + lane] = mine / (wsum + 1e-20f);
+  if (wave == 0 && lane < top) wout[t * top + lane] = mine / (wsum + 1e-20f);
 }
 
 // ---- combine: out[t] = sum_j w[t,j] * (rowidx[t,j] >= 0 ? rows[rowidx[t,j]] : h[t]) ------
@@ -436,8 +453,10 @@ extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h,
 extern "C" void seq_launch_moe_route(int* idx, float* w, int* rowidx, const float* z, const void* h,
                                      const float* router, const float* corr, int T_, int N, int W, int top,
                                      int gc, int gk, int E, int is_f32, hipStream_t st) {
-  DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_route_kernel<T>, dim3(T_), dim3(WAVE), 0, st, idx, w, rowidx, z,
-                                        (const T*)h, router, corr, N, W, top, gc, gk, E, T_);)
+  const int vec = (h != nullptr && W % 8 == 0 && aligned16(h) && aligned16(router)) ? 1 : 0;
+  const int threads = h != nullptr ? 256 : WAVE;
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_route_kernel<T>, dim3(T_), dim3(threads), 0, st, idx, w, rowidx, z,
+                                        (const T*)h, router, corr, N, W, top, gc, gk, E, T_, vec);)
 }
 
 extern "C" void seq_launch_moe_combine(void* out, const void* rows, const void* h, const int* rowidx,
