@@ -492,8 +492,14 @@ class RoutedExperts(nn.Module):
     Few rows: every expert runs on every row as two batched GEMMs (the weights
     stream from memory once either way, and shapes do not depend on the
     routing). Many rows: rows are sorted by expert and each expert runs on its
-    slice. Both end in one weighted gather that sums a row's choices in a
+    slice, which costs a host round trip and a few launches per expert; the
+    switch is made where the all-experts form's surplus arithmetic outweighs
+    that. Both end in one weighted gather that sums a row's choices in a
     fixed order, so a row's result does not depend on the batch around it."""
+
+    # surplus multiply-adds of the all-experts form above which rows are sorted
+    # by expert instead (about half a millisecond of matrix-core time)
+    DENSE_SURPLUS_FLOPS = 3.0e11
 
     def __init__(self, spec: RoutedExpertsSpec, hidden: int, dtype):
         super().__init__()
@@ -510,7 +516,7 @@ class RoutedExperts(nn.Module):
         sp = self.spec
         T, W = h.shape
         E, top = sp.experts, sp.top
-        dense = T <= 8 * E
+        dense = (E - min(top, E)) * T * 6.0 * W * sp.ff <= self.DENSE_SURPLUS_FLOPS
         idx, w, rowidx = ops.moe_route_rows(h, self.router, self.correction, top, sp.group_count, sp.group_keep,
                                             E, dense)
         if dense:

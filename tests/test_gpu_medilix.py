@@ -40,9 +40,9 @@ def test_fp32_mixed_schedule_matches_oracle(tmp_path, cfg, seed, rank):
     assert eng.kv.slots.num_free == eng.kv.slots.num_slots
 
 
-def test_fp32_long_decode_and_many_rows(tmp_path):
-    """150 single-token steps after a short prompt, and one portion long
-    enough for the sorted expert path."""
+def test_fp32_long_decode_and_sorted_experts(tmp_path, monkeypatch):
+    """150 single-token steps after a short prompt, and whole portions with the
+    experts' rows sorted by expert instead of every expert on every row."""
     cfg = CFG_A
     w = write_model(str(tmp_path), cfg, seed=1)
     eng = gpu_engine(tmp_path, "float32")
@@ -51,6 +51,11 @@ def test_fp32_long_decode_and_many_rows(tmp_path):
     got = run_schedule(eng, [[("x", 4)]] + [[("x", 1)]] * 150, {"x": p})["x"]
     torch.testing.assert_close(got.double().cpu(), want, rtol=1e-4, atol=5e-4)
     got = run_schedule(eng, [[("y", 154)]], {"y": p})["y"]
+    torch.testing.assert_close(got.double().cpu(), want, rtol=1e-4, atol=5e-4)
+    from kllms_amd.models.mixers import RoutedExperts
+
+    monkeypatch.setattr(RoutedExperts, "DENSE_SURPLUS_FLOPS", -1.0)
+    got = run_schedule(eng, [[("z", 100)], [("z", 1)], [("z", 53)]], {"z": p})["z"]
     torch.testing.assert_close(got.double().cpu(), want, rtol=1e-4, atol=5e-4)
 
 

@@ -273,11 +273,14 @@ def test_clamped_glu_both_clamps_active():
     check(mod(h.float()), O.dense_ff(h, w, "l0.mlp.", mlp))
 
 
-@pytest.mark.parametrize("name,T", [("moe", 7), ("moe", 90), ("moe_plain", 5), ("moe_plain", 70)])
-def test_routed_experts(name, T):
-    """Few rows (every expert on every row) and many rows (rows sorted by
-    expert) against the per-token oracle; corrections are negative, so an
-    excluded group must count as minus infinity, not 0."""
+@pytest.mark.parametrize("name,T,sorted_form", [("moe", 7, False), ("moe", 90, True), ("moe", 33, True),
+                                               ("moe_plain", 5, False), ("moe_plain", 70, True)])
+def test_routed_experts(name, T, sorted_form, monkeypatch):
+    """Both forms (every expert on every row; rows sorted by expert) against
+    the per-token oracle; corrections are negative, so an excluded group must
+    count as minus infinity, not 0."""
+    if sorted_form:
+        monkeypatch.setattr(RoutedExperts, "DENSE_SURPLUS_FLOPS", -1.0)
     mlp = MLPS[name]
     r = mlp["router"]
     w = O.random_weights({"vocab": 8, "width": 24, "norm": {"eps": EPS, "groups": 1},
