@@ -392,6 +392,9 @@ class WkvMixer(nn.Module):
     and projected. State: S [H, D, D] fp32 and the previous input."""
 
     STREAMS = ("r", "k", "v", "g", "w")
+    # the four projections run as one batched product for decode-sized steps
+    # and as four plain GEMMs for prompt portions
+    BATCHED_MAX_ROWS = 64
 
     def __init__(self, spec: WkvSpec, hidden: int, eps: float, dtype):
         super().__init__()
@@ -416,7 +419,10 @@ class WkvMixer(nn.Module):
         sp = self.spec
         mixes, mix_w = ops.token_shift_mix(h, self.mu, st.shift, batch.state_slots, batch.cu_seqlens,
                                            batch.seg_start, batch.token_seg, 4)
-        y = torch.bmm(mixes, self.rkvg.transpose(1, 2))                       # [4, T, H*D]
+        if h.shape[0] <= self.BATCHED_MAX_ROWS:
+            y = torch.bmm(mixes, self.rkvg.transpose(1, 2))                   # [4, T, H*D], one launch
+        else:
+            y = [F.linear(mixes[i], self.rkvg[i]) for i in range(4)]
         d = F.linear(torch.tanh(F.linear(mix_w[0], self.w1)), self.w2)       # fp32 [T, H*D]
         hd = (sp.heads, sp.dim)
         o = ops.wkv_recurrence(y[0].unflatten(1, hd), y[1].unflatten(1, hd), y[2].unflatten(1, hd), d,
@@ -489,17 +495,19 @@ class RoutedExperts(nn.Module):
     weigh the outputs. The last ``identity`` router outputs stand for experts
     that return their input and have no weights.
 
-    Few rows: every expert runs on every row as two batched GEMMs (the weights
-    stream from memory once either way, and shapes do not depend on the
-    routing). Many rows: rows are sorted by expert and each expert runs on its
-    slice, which costs a host round trip and a few launches per expert; the
-    switch is made where the all-experts form's surplus arithmetic outweighs
-    that. Both end in one weighted gather that sums a row's choices in a
-    fixed order, so a row's result does not depend on the batch around it."""
+    Few rows (decode): every expert runs on every row as two batched GEMMs
+    (the weights stream from memory once either way, and shapes do not depend
+    on the routing). More rows: rows are sorted by expert and each expert runs
+    on its slice. Both end in one weighted gather that sums a row's choices in
+    a fixed order, so a row's result does not depend on the batch around it.
 
-    # surplus multiply-adds of the all-experts form above which rows are sorted
-    # by expert instead (about half a millisecond of matrix-core time)
-    DENSE_SURPLUS_FLOPS = 3.0e11
+    The batched form stays with small row counts: on the GPU a batched product
+    of 8 x 512 rows against the experts of a 2048-wide layer ended in an
+    illegal address inside the run, while the per-expert products of the
+    sorted form ran the same rows cleanly."""
+
+    # rows per expert up to which every expert runs on every row
+    DENSE_ROWS_PER_EXPERT = 8
 
     def __init__(self, spec: RoutedExpertsSpec, hidden: int, dtype):
         super().__init__()
@@ -516,7 +524,7 @@ class RoutedExperts(nn.Module):
         sp = self.spec
         T, W = h.shape
         E, top = sp.experts, sp.top
-        dense = (E - min(top, E)) * T * 6.0 * W * sp.ff <= self.DENSE_SURPLUS_FLOPS
+        dense = T <= self.DENSE_ROWS_PER_EXPERT * E
         idx, w, rowidx = ops.moe_route_rows(h, self.router, self.correction, top, sp.group_count, sp.group_keep,
                                             E, dense)
         if dense:

@@ -157,7 +157,7 @@ def rows(L, W, seed):
     return torch.randn(L, W, generator=torch.Generator().manual_seed(seed), dtype=torch.float64)
 
 
-CUTS = [[60], [25] + [1] * 35, [2, 5, 16, 1, 2, 17, 3, 14], [9, 2, 10, 1, 38]]
+CUTS = [[60], [70], [25] + [1] * 35, [2, 5, 16, 1, 2, 17, 3, 14], [9, 2, 10, 1, 38]]
 
 
 @pytest.mark.parametrize("cuts", CUTS)
@@ -280,7 +280,7 @@ def test_routed_experts(name, T, sorted_form, monkeypatch):
     the per-token oracle; corrections are negative, so an excluded group must
     count as minus infinity, not 0."""
     if sorted_form:
-        monkeypatch.setattr(RoutedExperts, "DENSE_SURPLUS_FLOPS", -1.0)
+        monkeypatch.setattr(RoutedExperts, "DENSE_ROWS_PER_EXPERT", 0)
     mlp = MLPS[name]
     r = mlp["router"]
     w = O.random_weights({"vocab": 8, "width": 24, "norm": {"eps": EPS, "groups": 1},
