@@ -506,8 +506,10 @@ class RoutedExperts(nn.Module):
     illegal address inside the run, while the per-expert products of the
     sorted form ran the same rows cleanly."""
 
-    # rows per expert up to which every expert runs on every row
-    DENSE_ROWS_PER_EXPERT = 8
+    # every expert runs on every row for steps of at most this many rows, and
+    # at most this many (expert, row) pairs
+    DENSE_MAX_ROWS = 64
+    DENSE_MAX_PAIRS = 512
 
     def __init__(self, spec: RoutedExpertsSpec, hidden: int, dtype):
         super().__init__()
@@ -524,7 +526,7 @@ class RoutedExperts(nn.Module):
         sp = self.spec
         T, W = h.shape
         E, top = sp.experts, sp.top
-        dense = T <= self.DENSE_ROWS_PER_EXPERT * E
+        dense = T <= self.DENSE_MAX_ROWS and E * T <= self.DENSE_MAX_PAIRS
         idx, w, rowidx = ops.moe_route_rows(h, self.router, self.correction, top, sp.group_count, sp.group_keep,
                                             E, dense)
         if dense:

@@ -54,7 +54,7 @@ def test_fp32_long_decode_and_sorted_experts(tmp_path, monkeypatch):
     torch.testing.assert_close(got.double().cpu(), want, rtol=1e-4, atol=5e-4)
     from kllms_amd.models.mixers import RoutedExperts
 
-    monkeypatch.setattr(RoutedExperts, "DENSE_ROWS_PER_EXPERT", 0)
+    monkeypatch.setattr(RoutedExperts, "DENSE_MAX_ROWS", 0)
     got = run_schedule(eng, [[("z", 100)], [("z", 1)], [("z", 53)]], {"z": p})["z"]
     torch.testing.assert_close(got.double().cpu(), want, rtol=1e-4, atol=5e-4)
 

@@ -280,7 +280,7 @@ def test_routed_experts(name, T, sorted_form, monkeypatch):
     the per-token oracle; corrections are negative, so an excluded group must
     count as minus infinity, not 0."""
     if sorted_form:
-        monkeypatch.setattr(RoutedExperts, "DENSE_ROWS_PER_EXPERT", 0)
+        monkeypatch.setattr(RoutedExperts, "DENSE_MAX_ROWS", 0)
     mlp = MLPS[name]
     r = mlp["router"]
     w = O.random_weights({"vocab": 8, "width": 24, "norm": {"eps": EPS, "groups": 1},
